@@ -3,11 +3,11 @@
 #include "common.h"
 
 // ---------------------------------------------------------------- embedding gather
-// out[row, :] = table[ids[row], :], widened to 32-bit (the residual stream).
+// out[row, :] = table[ids[row], :] * scale, widened to 32-bit (the residual stream) and scaled there.
 // Reference: src/backend/cuda/kernels/embedding.cu:26-37.
 template <typename TW>
 __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict__ ids,
-                             float* __restrict__ out, int width, int vocab) {
+                             float* __restrict__ out, int width, int vocab, float scale) {
     const int row = blockIdx.x;
     const int id = ids[row];
     float* dst = out + static_cast<size_t>(row) * width;
@@ -16,19 +16,31 @@ __global__ void embed_kernel(const TW* __restrict__ table, const int* __restrict
         return;
     }
     const TW* src = table + static_cast<size_t>(id) * width;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float(src[i]);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = scale == 1.0f ? to_float(src[i]) : to_float(src[i]) * scale;
+}
+
+// x *= scale, 32-bit
+__global__ void scale_f32_kernel(float* __restrict__ x, size_t total, float scale) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < total) x[i] *= scale;
+}
+
+extern "C" int celeg_scale_f32(float* x, size_t total, float scale, hipStream_t stream) {
+    if (total == 0) return 0;
+    hipLaunchKernelGGL(scale_f32_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream, x, total, scale);
+    return CELEG_LAUNCH_RESULT();
 }
 
 extern "C" int celeg_embed(const void* table, int table_dtype, const int* ids, float* out,
-                           int rows, int width, int vocab, hipStream_t stream) {
+                           int rows, int width, int vocab, float scale, hipStream_t stream) {
     if (rows <= 0) return 0;
     dim3 grid(rows), block(256);
     if (table_dtype == CELEG_F32)
         hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream,
-                           static_cast<const float*>(table), ids, out, width, vocab);
+                           static_cast<const float*>(table), ids, out, width, vocab, scale);
     else
         hipLaunchKernelGGL(embed_kernel<bf16>, grid, block, 0, stream,
-                           static_cast<const bf16*>(table), ids, out, width, vocab);
+                           static_cast<const bf16*>(table), ids, out, width, vocab, scale);
     return CELEG_LAUNCH_RESULT();
 }
 

@@ -70,7 +70,7 @@ Json CacheLayout::to_json() const {
     Json groups = Json::array();
     for (size_t g = 0; g < kv_groups.size(); ++g)
         groups.push(Json::object().set("kv_heads", kv_groups[g].kv_heads).set("head_dim", kv_groups[g].head_dim)
-                        .set("v_head_dim", kv_groups[g].value_dim())
+                        .set("v_head_dim", kv_groups[g].value_dim()).set("keys_only", kv_groups[g].keys_only)
                         .set("window", kv_groups[g].window ? Json(*kv_groups[g].window) : Json())
                         .set("layers", group_layers[g]));
     Json uses = Json::array();
@@ -92,7 +92,8 @@ CacheLayout CacheLayout::from_json(const Json& j) {
             need.kv_heads = static_cast<int>(g.get_int("kv_heads", 0));
             need.head_dim = static_cast<int>(g.get_int("head_dim", 0));
             need.v_head_dim = static_cast<int>(g.get_int("v_head_dim", 0));
-            if (need.v_head_dim == need.head_dim) need.v_head_dim = 0;
+            need.keys_only = g.get_bool("keys_only", false);
+            if (need.v_head_dim == need.head_dim || need.keys_only) need.v_head_dim = 0;
             if (!g["window"].is_null()) need.window = static_cast<int>(g["window"].as_int());
             out.kv_groups.push_back(need);
             out.group_layers.push_back(static_cast<int>(g.get_int("layers", 1)));
@@ -148,7 +149,7 @@ CacheManager::CacheManager(CacheLayout layout_, int page_tokens_, std::vector<in
         if (on_device_) {
             const size_t per_dim = static_cast<size_t>(n_pages[g] + 1) * grp.n_layers * need.kv_heads * page_tokens * itemsize;
             grp.k = DeviceBuffer(per_dim * need.head_dim, true);
-            grp.v = DeviceBuffer(per_dim * need.value_dim(), true);
+            if (!need.keys_only) grp.v = DeviceBuffer(per_dim * need.value_dim(), true);
             grp.table = DeviceBuffer(grp.table_host.size() * sizeof(int));
             CELEG_HIP(hipMemcpy(grp.table.ptr(), grp.table_host.data(), grp.table_host.size() * sizeof(int),
                                 hipMemcpyHostToDevice));

@@ -11,7 +11,7 @@
 //
 // Storage of a group: K [pages + 1, layers, kv_heads, page_tokens, head_dim] and V
 // [pages + 1, layers, kv_heads, v_head_dim, page_tokens] (transposed inside a page: the layout
-// the matrix-core attention kernel reads without shuffling).  The extra last page is never
+// the matrix-core attention kernel reads without shuffling); a keys-only group has no V.  The extra last page is never
 // handed out: rows that pad a batch to a fixed size write there.  Likewise the last slot
 // (null_slot) is never given to a request.
 //
@@ -55,14 +55,17 @@ private:
 };
 
 // Keys and values of every position, or of a trailing window of positions.  Values may have
-// another width than keys (v_head_dim; 0: the keys').
+// another width than keys (v_head_dim; 0: the keys'), or there may be none (keys_only: the mixer
+// reads its values out of the key rows, as an attention over compressed rows does).
 struct KVNeed {
     int kv_heads = 0, head_dim = 0;
     std::optional<int> window;
     int v_head_dim = 0;
-    int value_dim() const { return v_head_dim > 0 ? v_head_dim : head_dim; }
+    bool keys_only = false;
+    int value_dim() const { return keys_only ? 0 : v_head_dim > 0 ? v_head_dim : head_dim; }
     bool operator==(const KVNeed& o) const {
-        return kv_heads == o.kv_heads && head_dim == o.head_dim && window == o.window && value_dim() == o.value_dim();
+        return kv_heads == o.kv_heads && head_dim == o.head_dim && window == o.window && value_dim() == o.value_dim() &&
+               keys_only == o.keys_only;
     }
 };
 

@@ -58,7 +58,8 @@ std::string architecture_name(const Json& config) {
     const Json& archs = config["architectures"];
     if (archs.is_array() && archs.size() > 0 && archs[0].is_string()) return archs[0].as_string();
     if (config["model_type"].is_string()) return config["model_type"].as_string();
-    throw ConfigError("config.json names no architecture: neither 'architectures' nor 'model_type' is present");
+    if (config["architecture"].is_string()) return config["architecture"].as_string();
+    throw ConfigError("config.json names no architecture: none of 'architectures', 'model_type' and 'architecture' is present");
 }
 
 const Architecture& find_architecture(const Json& config) {
@@ -406,6 +407,213 @@ ModelSpec lfm2_build_spec(const Json& c) {
     return spec;
 }
 
+}  // namespace
+
+// ---------------------------------------------------------------------------- Regipel
+// A decoder whose config.json describes every layer by itself:
+//   {"architecture": "Regipel", "vocab", "width", "norm": {"eps"}, "embedding": {"scale"},
+//    "logit_scale", "streams" (absent: one residual stream and plain pre-norm sums),
+//    "loop": {"start", "stop", "times"} (layers start..stop-1 run `times` times in a row with the
+//    same weights and a cache of their own each time), "max_context" (an engine limit; optional),
+//    "layers": [{"type": "latent_attention",
+//                "mixer": {"heads", "dim", "rot_dim", "vdim", "kv_rank", "scale", "rot": {"base", "dims"}},
+//                "mlp": null | {"kind": "moe", "expert": {"ff"}, "router": {"experts", "top"}}}]}
+// Norm weights are stored around zero (the factor is 1 + w); the output head is the embedding
+// table itself, the logits multiplied by logit_scale.
+// Tensors: embed, final.norm, l<i>.norm1, l<i>.norm2, l<i>.mix.{q,dkv,dkv.norm,uk,uv,sink,g,o},
+// l<i>.mlp.router, l<i>.mlp.e<j>.{gate,up,down}, l<i>.hc<q>.{in,out,mix} (q = 1: mixer, 2: feed-forward).
+namespace {
+
+const Json& regipel_object(const Json& parent, const std::string& key, const std::string& where) {
+    const Json& v = parent[key];
+    if (!v.is_object()) throw ConfigError("config.json: " + where + "'" + key + "' must be an object");
+    return v;
+}
+long long regipel_int(const Json& parent, const std::string& key, const std::string& where, long long least = 1) {
+    const Json& v = parent[key];
+    if (!v.is_int()) throw ConfigError("config.json: " + where + "'" + key + "' must be an integer, got " + v.dump());
+    if (v.as_int() < least)
+        throw ConfigError("config.json: " + where + "'" + key + "' must be at least " + std::to_string(least) + ", got " + v.dump());
+    return v.as_int();
+}
+double regipel_number(const Json& parent, const std::string& key, const std::string& where) {
+    const Json& v = parent[key];
+    if (!v.is_number()) throw ConfigError("config.json: " + where + "'" + key + "' must be a number, got " + v.dump());
+    return v.as_double();
+}
+
+Json regipel_read_config(const Json& raw, const TensorShapes*) {
+    if (!raw.is_object()) throw ConfigError("config.json is not an object");
+    Json out = Json::object();
+    out.set("architecture", "Regipel");
+    out.set("vocab", regipel_int(raw, "vocab", ""));
+    out.set("width", regipel_int(raw, "width", ""));
+    const double eps = regipel_number(regipel_object(raw, "norm", ""), "eps", "norm.");
+    if (!(eps > 0)) throw ConfigError("config.json: 'norm.eps' must be positive");
+    out.set("norm", Json::object().set("eps", eps));
+    double embedding_scale = 1.0, logit_scale = 1.0;
+    if (!raw["embedding"].is_null()) embedding_scale = regipel_number(regipel_object(raw, "embedding", ""), "scale", "embedding.");
+    if (!raw["logit_scale"].is_null()) logit_scale = regipel_number(raw, "logit_scale", "");
+    out.set("embedding", Json::object().set("scale", embedding_scale)).set("logit_scale", logit_scale);
+    out.set("streams", raw["streams"].is_null() ? Json() : Json(regipel_int(raw, "streams", "")));
+    if (!out["streams"].is_null() && out["streams"].as_int() > 8) throw ConfigError("config.json: 'streams' may be at most 8");
+    out.set("max_context", raw["max_context"].is_null() ? 131072LL : regipel_int(raw, "max_context", ""));
+    if (!raw["layers"].is_array() || raw["layers"].size() == 0) throw ConfigError("config.json: 'layers' must be a list of layers");
+    Json layers = Json::array();
+    int i = 0;
+    for (const Json& l : raw["layers"].items()) {
+        const std::string where = "layers[" + std::to_string(i++) + "].";
+        if (!l.is_object()) throw ConfigError("config.json: " + where + " must be an object");
+        const std::string type = l.get_string("type", "");
+        if (type != "latent_attention")
+            throw ConfigError("config.json: " + where + "'type' is '" + type + "'; known types are ['latent_attention']");
+        const Json& m = regipel_object(l, "mixer", where);
+        const std::string mw = where + "mixer.";
+        Json mixer = Json::object();
+        for (const char* key : {"heads", "dim", "vdim", "kv_rank"}) mixer.set(key, regipel_int(m, key, mw));
+        const long long rot_dim = regipel_int(m, "rot_dim", mw, 0);
+        mixer.set("rot_dim", rot_dim);
+        mixer.set("scale", regipel_number(m, "scale", mw));
+        if (rot_dim > 0) {
+            const Json& rot = regipel_object(m, "rot", mw);
+            const long long dims = regipel_int(rot, "dims", mw + "rot.", 0);
+            const double base = regipel_number(rot, "base", mw + "rot.");
+            if (dims % 2 || dims > rot_dim) throw ConfigError("config.json: " + mw + "'rot.dims' must be even and at most 'rot_dim'");
+            if (!(base > 0)) throw ConfigError("config.json: " + mw + "'rot.base' must be positive");
+            mixer.set("rot", Json::object().set("base", base).set("dims", dims));
+        } else {
+            mixer.set("rot", Json());
+        }
+        mixer.set("sink", m.get_bool("sink", true)).set("gate", m.get_bool("gate", true));
+        Json mlp;
+        if (!l["mlp"].is_null()) {
+            const Json& f = regipel_object(l, "mlp", where);
+            const std::string fw = where + "mlp.";
+            const std::string kind = f.get_string("kind", "");
+            if (kind != "moe") throw ConfigError("config.json: " + fw + "'kind' is '" + kind + "'; known kinds are ['moe']");
+            const Json& router = regipel_object(f, "router", fw);
+            const long long experts = regipel_int(router, "experts", fw + "router."), top = regipel_int(router, "top", fw + "router.");
+            if (top > experts) throw ConfigError("config.json: " + fw + "'router.top' exceeds 'router.experts'");
+            if (experts > 512) throw ConfigError("config.json: " + fw + "'router.experts' may be at most 512");
+            mlp = Json::object().set("kind", kind)
+                      .set("expert", Json::object().set("ff", regipel_int(regipel_object(f, "expert", fw), "ff", fw + "expert.")))
+                      .set("router", Json::object().set("experts", experts).set("top", top));
+        }
+        layers.push(Json::object().set("type", type).set("mixer", mixer).set("mlp", mlp));
+    }
+    out.set("layers", layers);
+    const long long n_layers = static_cast<long long>(layers.size());
+    long long start = 0, stop = 0, times = 1;
+    if (!raw["loop"].is_null()) {
+        const Json& loop = regipel_object(raw, "loop", "");
+        start = regipel_int(loop, "start", "loop.", 0);
+        stop = regipel_int(loop, "stop", "loop.", 0);
+        times = regipel_int(loop, "times", "loop.", 0);
+        if (start > stop || stop > n_layers)
+            throw ConfigError("config.json: 'loop' must satisfy 0 <= start <= stop <= " + std::to_string(n_layers));
+    }
+    out.set("loop", Json::object().set("start", start).set("stop", stop).set("times", times));
+    for (const char* key : {"bos_token_id", "eos_token_id"})
+        if (!raw[key].is_null()) out.set(key, raw[key]);
+    return out;
+}
+
+ModelSpec regipel_build_spec(const Json& c) {
+    const long long W = c["width"].as_int();
+    const double eps = c["norm"]["eps"].as_double();
+    const bool hyper = !c["streams"].is_null();
+    const long long S = hyper ? c["streams"].as_int() : 1;
+    auto norm = [&](const std::string& name) {
+        PartSpec p;
+        p.kind = "rmsnorm";
+        p.params = Json::object().set("width", W).set("eps", eps).set("weight_offset", 1.0);
+        p.tensors = {{"weight", name}};
+        return p;
+    };
+    auto link = [&](const std::string& prefix) {
+        PartSpec p;
+        p.kind = "hyper_link";
+        p.params = Json::object().set("streams", S);
+        p.tensors = {{"in", prefix + ".in"}, {"out", prefix + ".out"}, {"mix", prefix + ".mix"}};
+        return p;
+    };
+    ModelSpec spec;
+    int i = 0;
+    for (const Json& l : c["layers"].items()) {
+        const std::string p = "l" + std::to_string(i) + ".";
+        const Json& m = l["mixer"];
+        LayerSpec layer;
+        layer.arrangement = hyper ? "hyper_connections" : "pre_norm";
+        layer.mixer.kind = "latent_attention";
+        layer.mixer.params = Json::object().set("width", W).set("heads", m["heads"]).set("dim", m["dim"])
+                                 .set("rot_dim", m["rot_dim"]).set("vdim", m["vdim"]).set("kv_rank", m["kv_rank"])
+                                 .set("scale", m["scale"]).set("eps", eps).set("sink", m["sink"]).set("gate", m["gate"]);
+        if (!m["rot"].is_null() && m["rot"]["dims"].as_int() > 0) {
+            PartSpec rope;
+            rope.kind = "rope";
+            rope.params = Json::object().set("theta", m["rot"]["base"]).set("rotary_dim", m["rot"]["dims"])
+                              .set("head_dim", m["rot_dim"]).set("pairing", "neighbours");
+            layer.mixer.params.set("position", rope.to_json());
+        }
+        layer.mixer.tensors = {{"q", p + "mix.q"},   {"dkv", p + "mix.dkv"}, {"dkv_norm", p + "mix.dkv.norm"},
+                               {"uk", p + "mix.uk"}, {"uv", p + "mix.uv"},   {"o", p + "mix.o"}};
+        if (m["sink"].as_bool()) layer.mixer.tensors.emplace_back("sink", p + "mix.sink");
+        if (m["gate"].as_bool()) layer.mixer.tensors.emplace_back("g", p + "mix.g");
+        layer.mixer_norm = norm(p + "norm1");
+        if (hyper) layer.mixer_link = link(p + "hc1");
+        if (l["mlp"].is_null()) {
+            layer.ffn.kind = "none";
+            layer.ffn_norm.kind = "identity";
+        } else {
+            const Json& f = l["mlp"];
+            const long long experts = f["router"]["experts"].as_int();
+            layer.ffn.kind = "routed_experts";
+            layer.ffn.params = Json::object().set("width", W).set("ff", f["expert"]["ff"]).set("experts", experts)
+                                   .set("top", f["router"]["top"]).set("score", "sigmoid").set("renormalize", false)
+                                   .set("weight_on", "input");
+            layer.ffn.tensors = {{"router", p + "mlp.router"}};
+            for (long long e = 0; e < experts; ++e) {
+                const std::string ep = p + "mlp.e" + std::to_string(e) + ".", n = std::to_string(e);
+                layer.ffn.tensors.emplace_back("gate." + n, ep + "gate");
+                layer.ffn.tensors.emplace_back("up." + n, ep + "up");
+                layer.ffn.tensors.emplace_back("down." + n, ep + "down");
+            }
+            layer.ffn_norm = norm(p + "norm2");
+            if (hyper) layer.ffn_link = link(p + "hc2");
+        }
+        spec.layers.push_back(std::move(layer));
+        ++i;
+    }
+    const int n_layers = i;
+    const int start = static_cast<int>(c["loop"]["start"].as_int()), stop = static_cast<int>(c["loop"]["stop"].as_int());
+    const int times = static_cast<int>(c["loop"]["times"].as_int());
+    for (int l = 0; l < start; ++l) spec.order.push_back(RunStep{l, {}});
+    for (int pass = 0; pass < times; ++pass)
+        for (int l = start; l < stop; ++l) spec.order.push_back(RunStep{l, {}});
+    for (int l = stop; l < n_layers; ++l) spec.order.push_back(RunStep{l, {}});
+    spec.architecture = "Regipel";
+    spec.vocab_size = static_cast<int>(c["vocab"].as_int());
+    spec.hidden_size = static_cast<int>(W);
+    spec.max_context = static_cast<int>(c["max_context"].as_int());
+    spec.streams = static_cast<int>(S);
+    spec.embedding.kind = "embedding";
+    spec.embedding.params = Json::object().set("vocab", c["vocab"]).set("width", W).set("scale", c["embedding"]["scale"]);
+    spec.embedding.tensors = {{"table", "embed"}};
+    spec.head.kind = "tied_head";
+    spec.head.params = Json::object().set("vocab", c["vocab"]).set("width", W).set("scale", c["logit_scale"]);
+    spec.final_norm = norm("final.norm");
+    if (c["eos_token_id"].is_array())
+        for (const Json& e : c["eos_token_id"].items()) spec.eos_token_ids.push_back(static_cast<int>(e.as_int()));
+    else if (c["eos_token_id"].is_int())
+        spec.eos_token_ids.push_back(static_cast<int>(c["eos_token_id"].as_int()));
+    if (c["bos_token_id"].is_int()) spec.bos_token_id = static_cast<int>(c["bos_token_id"].as_int());
+    spec.validate();
+    return spec;
+}
+
+}  // namespace
+
+namespace {
 void register_builtin() {
     Architecture lfm2;
     lfm2.name = "Lfm2ForCausalLM";
@@ -415,6 +623,13 @@ void register_builtin() {
     std::lock_guard<std::mutex> guard(table_lock());
     table()["Lfm2ForCausalLM"] = lfm2;
     table()["lfm2"] = lfm2;
+    Architecture regipel;
+    regipel.name = "Regipel";
+    regipel.aliases = {"regipel"};
+    regipel.read_config = regipel_read_config;
+    regipel.build_spec = regipel_build_spec;
+    table()["Regipel"] = regipel;
+    table()["regipel"] = regipel;
 }
 
 }  // namespace

@@ -14,7 +14,8 @@
 extern "C" {
 // elementwise.hip
 int celeg_embed(const void* table, int table_dtype, const int* ids, float* out, int rows, int width, int vocab,
-                hipStream_t stream);
+                float scale, hipStream_t stream);
+int celeg_scale_f32(float* x, size_t total, float scale, hipStream_t stream);
 int celeg_rmsnorm(void* x, int x_dtype, const void* delta, int delta_dtype, const float* w, void* out, int out_dtype,
                   const int* rows, int n_rows, int width, float eps, int write_back, hipStream_t stream);
 int celeg_swiglu(const void* gu, void* out, int dtype, int rows, int ff, hipStream_t stream);
@@ -26,6 +27,35 @@ int celeg_step_prologue(int* table, int stride, int n_slots, const int* updates,
 int celeg_resolve_tokens(int* token_ids, const int* token_slot, const int* last_tokens, int n, hipStream_t stream);
 int celeg_fold_weight(const void* w, const float* scale, void* out, int rows, int K, int packed, hipStream_t stream);
 int celeg_zero_words(void* p, size_t words, hipStream_t stream);
+// hyper.hip
+int celeg_streams_spread(const float* h, float* xs, int rows, int streams, int width, hipStream_t stream);
+int celeg_streams_sum(const float* xs, float* h, int rows, int streams, int width, hipStream_t stream);
+int celeg_hyper_step(float* xs, const void* y, int y_dtype, const float* mix, const float* out_w, const float* in_w,
+                     const float* w, float eps, void* normed, int out_dtype, int rows, int streams, int width,
+                     hipStream_t stream);
+// latent.hip
+int celeg_latent_prepare(void* proj, int ld, int dtype, int q_off, int dkv_off, int heads, int dim, int rot, int rank,
+                         const float* weight, float eps, const float* inv_freq, int rotary, int pairing,
+                         const int* positions, const int* token_slot, const int* table, int table_stride, void* pool,
+                         int n_layers, int layer, int page_tokens, int write, int n_tokens, hipStream_t stream);
+int celeg_headwise_linear(const void* x, int ldx, int x_head, const void* w, int dtype, int heads, int N, int K, void* out,
+                          int ldo, int o_head, int tail, const void* gate, int ldg, int rows, hipStream_t stream);
+int celeg_latent_attention(const void* q, int ldq, const void* pool, int dtype, const int* table, int table_stride,
+                           const int* token_slot, const int* positions, const float* sink, void* out, int ldo,
+                           int n_tokens, int heads, int rank, int rot, int page_tokens, int n_layers, int layer,
+                           float scale, hipStream_t stream);
+// moe.hip
+int celeg_moe_route(const float* logits, int rows, int experts, int top, int score, int renorm, int* ids, float* weights,
+                    hipStream_t stream);
+int celeg_moe_tile_rows();
+int celeg_moe_plan(const int* ids, int n, int experts, int* offsets, int* place_of, int* entry_at, int* tile_expert,
+                   int* tile_row0, int* n_tiles, hipStream_t stream);
+int celeg_moe_gather(const void* x, int dtype, const int* entry_at, const float* weights, void* a, int n, int top, int width,
+                     hipStream_t stream);
+int celeg_moe_product(const void* a, const void* w, void* out, int dtype, int N, int K, int gated, const int* offsets,
+                      const int* tile_expert, const int* tile_row0, const int* n_tiles, int max_tiles, hipStream_t stream);
+int celeg_moe_combine(const void* y, int dtype, const int* place_of, const float* weights, void* out, int rows, int top,
+                      int width, hipStream_t stream);
 // gemm_f32.hip
 int celeg_gemm_f32(const float* X, int ldx, const float* W, int ldw, const float* bias, float* Y, int ldy, int M,
                    int N, int K, hipStream_t stream);

@@ -14,7 +14,13 @@ namespace celeg {
 Model::Model(ModelSpec s) : spec(std::move(s)) {
     spec.validate();
     embedding_ = build_as<Embedding>("embedding", spec.embedding);
-    for (const LayerSpec& layer : spec.layers) blocks_.push_back(build_block(layer));
+    for (const LayerSpec& layer : spec.layers) {
+        blocks_.push_back(build_block(layer));
+        if (blocks_.back()->streams() != spec.streams)
+            throw SpecError("layer " + std::to_string(blocks_.size() - 1) + " ('" + layer.arrangement + "') works on " +
+                            std::to_string(blocks_.back()->streams()) + " residual stream(s), the model keeps " +
+                            std::to_string(spec.streams));
+    }
     final_norm_ = build_as<Norm>("norm", spec.final_norm);
     head_ = build_as<Head>("head", spec.head);
     resolve_cache_sharing();
@@ -154,9 +160,25 @@ Tensor Model::forward(const StepBatch& batch, Runtime& rt) {
     rt.flush_prologue();      // (an embedding that said it would and did not)
     rt.mark("embedding");
     Tensor delta;
+    // several residual streams: every stream starts as the embedding's rows, the blocks work on
+    // [T, streams * width], and what follows the blocks sees the sum of the streams
+    const int S = spec.streams;
+    Tensor hs = h;
+    if (S > 1) {
+        hs = rt.ws.buf("hidden_streams", DType::F32, {T, S * width});
+        rt.ops.streams_spread(h, hs, S);
+    }
     for (size_t i = 0; i < spec.order.size(); ++i) {
-        delta = blocks_[static_cast<size_t>(spec.order[i].layer)]->forward(h, delta, batch, caches_[i], rt);
-        if (rt.after_layer) rt.after_layer(static_cast<int>(i), h, delta.defined() ? &delta : nullptr);
+        delta = blocks_[static_cast<size_t>(spec.order[i].layer)]->forward(hs, delta, batch, caches_[i], rt);
+        if (rt.after_layer) {
+            if (S > 1) rt.ops.streams_sum(hs, h, S);
+            rt.after_layer(static_cast<int>(i), h, delta.defined() ? &delta : nullptr);
+        }
+    }
+    if (S > 1) {
+        rt.ops.streams_sum(hs, h, S);
+        rt.stream_stat_blocks = 0;
+        rt.stream_has_bf16 = false;
     }
     Tensor logits = rt.ws.buf("logits", DType::F32, {R, vocab});
     if (R == 0) return logits;

@@ -51,6 +51,8 @@ const char* path_name(Path p) {
         case Path::AttentionDecodeFresh: return "attention_decode_fresh";
         case Path::AttentionRows: return "attention_rows";
         case Path::AttentionGeneral: return "attention_general";
+        case Path::AttentionLatent: return "attention_latent";
+        case Path::RoutedExperts: return "routed_experts";
         case Path::LinearF32: return "linear_f32";
         case Path::LinearLibrary: return "linear_library";
         case Path::LinearStandIn: return "linear_stand_in";
@@ -79,12 +81,207 @@ static int hint_of(const StepBatch& batch, const KVView& kv) {
 }
 
 // ---------------------------------------------------------------------------- row-wise
-void Ops::embed(const Tensor& table, const int* token_ids, const Tensor& out) {
+void Ops::embed(const Tensor& table, const int* token_ids, const Tensor& out, float scale) {
     dev(table, "table");
     dev(out, "out", DType::F32);
     need(table.ndim == 2 && out.ndim == 2 && table.shape[1] == out.shape[1] && table.contiguous(), "embed: shapes do not fit");
     kernel_check(celeg_embed(table.data, dt(table, "table"), token_ids, out.as<float>(), static_cast<int>(out.shape[0]),
-                             static_cast<int>(out.shape[1]), static_cast<int>(table.shape[0]), stream), "embed");
+                             static_cast<int>(out.shape[1]), static_cast<int>(table.shape[0]), scale, stream), "embed");
+}
+
+void Ops::scale(const Tensor& x, float factor) {
+    dev(x, "x", DType::F32);
+    kernel_check(celeg_scale_f32(x.as<float>(), static_cast<size_t>(x.numel()), factor, stream), "scale");
+}
+
+// ---------------------------------------------------------------------------- several residual streams
+void Ops::streams_spread(const Tensor& h, const Tensor& xs, int streams) {
+    dev(h, "h", DType::F32);
+    dev(xs, "xs", DType::F32);
+    need(h.ndim == 2 && xs.ndim == 2 && streams > 0 && xs.shape[0] == h.shape[0] && xs.shape[1] == streams * h.shape[1],
+         "streams_spread: xs must be [rows, streams * width]");
+    kernel_check(celeg_streams_spread(h.as<float>(), xs.as<float>(), static_cast<int>(h.shape[0]), streams,
+                                      static_cast<int>(h.shape[1]), stream), "streams_spread");
+}
+
+void Ops::streams_sum(const Tensor& xs, const Tensor& h, int streams) {
+    dev(h, "h", DType::F32);
+    dev(xs, "xs", DType::F32);
+    need(h.ndim == 2 && xs.ndim == 2 && streams > 0 && xs.shape[0] == h.shape[0] && xs.shape[1] == streams * h.shape[1],
+         "streams_sum: xs must be [rows, streams * width]");
+    kernel_check(celeg_streams_sum(xs.as<float>(), h.as<float>(), static_cast<int>(h.shape[0]), streams,
+                                   static_cast<int>(h.shape[1]), stream), "streams_sum");
+}
+
+void Ops::hyper_step(const Tensor& xs, int streams, const Tensor* y, const Tensor* mix, const Tensor* out_w,
+                     const Tensor* in_w, const Tensor* weight, float eps, const Tensor* normed) {
+    dev(xs, "xs", DType::F32);
+    need(xs.ndim == 2 && streams > 0 && streams <= 8 && xs.shape[1] % streams == 0, "hyper_step: xs must be [rows, streams * width] with at most 8 streams");
+    const long long rows = xs.shape[0], width = xs.shape[1] / streams;
+    need(width <= 16384, "hyper_step: rows of more than 16,384 values do not fit the kernel's row buffer");
+    if (y) {
+        dev(*y, "y");
+        need(mix && out_w, "hyper_step: a sub-layer output needs its mix and out weights");
+        dev(*mix, "mix", DType::F32);
+        dev(*out_w, "out", DType::F32);
+        need(y->ndim == 2 && y->contiguous() && y->shape[0] == rows && y->shape[1] == width && mix->numel() == streams * streams &&
+                 out_w->numel() == streams, "hyper_step: y [rows, width], mix [streams, streams], out [streams]");
+    }
+    if (in_w) {
+        dev(*in_w, "in", DType::F32);
+        need(normed != nullptr, "hyper_step: the mixture needs a place");
+        dev(*normed, "normed");
+        need(in_w->numel() == streams && normed->ndim == 2 && normed->contiguous() && normed->shape[0] == rows &&
+                 normed->shape[1] == width, "hyper_step: in [streams], normed [rows, width]");
+        if (weight) {
+            dev(*weight, "weight", DType::F32);
+            need(weight->numel() == width, "hyper_step: the norm's weight must have the rows' width");
+        } else {
+            need(normed->dtype == DType::F32, "hyper_step: a mixture that is not normalised leaves in 32-bit");
+        }
+    }
+    kernel_check(celeg_hyper_step(xs.as<float>(), y ? y->data : nullptr, y ? dt(*y, "y") : 0, mix ? mix->as<float>() : nullptr,
+                                  out_w ? out_w->as<float>() : nullptr, in_w ? in_w->as<float>() : nullptr,
+                                  weight ? weight->as<float>() : nullptr, eps, normed ? normed->data : nullptr,
+                                  normed ? dt(*normed, "normed") : 0, static_cast<int>(rows), streams, static_cast<int>(width),
+                                  stream), "hyper_step");
+}
+
+// ---------------------------------------------------------------------------- latent attention
+static void latent_cache_fits(const Ops::LatentShape& s, const KVView& kv, DType dtype, const char* who) {
+    need(kv.k != nullptr && kv.kv_heads == 1 && kv.head_dim == s.rank + s.rot,
+         std::string(who) + ": the cache must hold one row of rank + rot values per token");
+    need(kv.dtype == dtype, std::string(who) + ": the cache and the rows differ in dtype");
+}
+
+void Ops::latent_prepare(const Tensor& proj, int q_off, int dkv_off, const LatentShape& s, const Tensor& norm_weight,
+                         float eps, const Tensor* inv_freq, int rotary_dim, int pairing, bool write, const StepBatch& batch,
+                         const KVView& kv) {
+    dev(proj, "proj");
+    dev(norm_weight, "norm_weight", DType::F32);
+    const int ld = rows_of(proj, "proj");
+    need(s.heads > 0 && s.dim > 0 && s.rot >= 0 && s.rank > 0, "latent_prepare: sizes must be positive");
+    need(proj.shape[0] == batch.n_tokens, "latent_prepare: one row per token of the step");
+    need(q_off >= 0 && q_off + static_cast<long long>(s.heads) * (s.dim + s.rot) <= proj.shape[1] && dkv_off >= 0 &&
+             dkv_off + s.rank + s.rot <= proj.shape[1], "latent_prepare: the queries or the compressed part lie outside the rows");
+    need(norm_weight.numel() == s.rank, "latent_prepare: the norm's weight must have `rank` entries");
+    need(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= s.rot, "latent_prepare: rotary_dim must be even and at most rot");
+    if (rotary_dim > 0) {
+        need(inv_freq != nullptr, "latent_prepare: a rotation needs its frequencies");
+        dev(*inv_freq, "inv_freq", DType::F32);
+        need(inv_freq->numel() == rotary_dim / 2, "latent_prepare: one frequency per rotated pair");
+    }
+    latent_cache_fits(s, kv, proj.dtype, "latent_prepare");
+    kernel_check(celeg_latent_prepare(proj.data, ld, dt(proj, "proj"), q_off, dkv_off, s.heads, s.dim, s.rot, s.rank,
+                                      norm_weight.as<float>(), eps, inv_freq && rotary_dim > 0 ? inv_freq->as<float>() : nullptr,
+                                      rotary_dim, pairing, batch.positions, batch.token_slot, kv.table, kv.table_stride, kv.k,
+                                      kv.n_layers, kv.layer, kv.page_tokens, write ? 1 : 0, batch.n_tokens, stream),
+                 "latent_prepare");
+}
+
+void Ops::headwise_linear(const Tensor& x, int x_head, const Tensor& w, const Tensor& out, int o_head, int tail,
+                          const Tensor* gate) {
+    dev(x, "x");
+    dev(w, "w", x.dtype);
+    dev(out, "out", x.dtype, false);
+    need(w.ndim == 3, "headwise_linear: w must be [heads, N, K]");
+    const long long heads = w.shape[0], N = w.shape[1], K = w.shape[2];
+    const int ldx = rows_of(x, "x"), ldo = rows_of(out, "out");
+    need(x.shape[0] == out.shape[0] && tail >= 0 && x_head >= K + tail && o_head >= N + tail &&
+             (heads - 1) * x_head + K + tail <= x.shape[1] && (heads - 1) * o_head + N + tail <= out.shape[1],
+         "headwise_linear: the heads do not fit the rows");
+    int ldg = 0;
+    if (gate) {
+        dev(*gate, "gate", x.dtype, false);
+        ldg = rows_of(*gate, "gate");
+        need(gate->shape[0] == x.shape[0] && gate->shape[1] == heads * N, "headwise_linear: gate must be [rows, heads * N]");
+    }
+    kernel_check(celeg_headwise_linear(x.data, ldx, x_head, w.data, dt(x, "x"), static_cast<int>(heads), static_cast<int>(N),
+                                       static_cast<int>(K), out.data, ldo, o_head, tail, gate ? gate->data : nullptr, ldg,
+                                       static_cast<int>(x.shape[0]), stream), "headwise_linear");
+}
+
+void Ops::latent_attention(const Tensor& q_lat, const Tensor& out, const LatentShape& s, float scale, const Tensor* sink,
+                           const StepBatch& batch, const KVView& kv) {
+    dev(q_lat, "q_lat");
+    dev(out, "out", q_lat.dtype);
+    const int D = s.rank + s.rot;
+    need(q_lat.ndim == 2 && q_lat.contiguous() && q_lat.shape[0] == batch.n_tokens && q_lat.shape[1] == static_cast<long long>(s.heads) * D,
+         "latent_attention: q_lat must be [rows, heads * (rank + rot)]");
+    need(out.ndim == 2 && out.shape[0] == batch.n_tokens && out.shape[1] == static_cast<long long>(s.heads) * s.rank,
+         "latent_attention: out must be [rows, heads * rank]");
+    need(s.rank <= 512, "latent_attention: a compressed row of more than 512 values does not fit the kernel's accumulators");
+    if (sink) {
+        dev(*sink, "sink", DType::F32);
+        need(sink->numel() == s.heads, "latent_attention: one sink per head");
+    }
+    latent_cache_fits(s, kv, q_lat.dtype, "latent_attention");
+    took(Path::AttentionLatent);
+    kernel_check(celeg_latent_attention(q_lat.data, static_cast<int>(q_lat.shape[1]), kv.k, dt(q_lat, "q_lat"), kv.table,
+                                        kv.table_stride, batch.token_slot, batch.positions, sink ? sink->as<float>() : nullptr,
+                                        out.data, static_cast<int>(out.shape[1]), batch.n_tokens, s.heads, s.rank, s.rot,
+                                        kv.page_tokens, kv.n_layers, kv.layer, scale, stream), "latent_attention");
+}
+
+// ---------------------------------------------------------------------------- routed experts
+Ops::RoutePlan Ops::moe_route(const Tensor& logits, int top, int score, bool renorm, Workspace& ws) {
+    dev(logits, "logits", DType::F32);
+    need(logits.ndim == 2, "moe_route: logits must be [rows, experts]");
+    const long long rows = logits.shape[0], experts = logits.shape[1];
+    need(experts > 0 && experts <= 512, "moe_route: between 1 and 512 experts");
+    need(top > 0 && top <= experts, "moe_route: `top` must be between 1 and the number of experts");
+    need(score == 0 || score == 1, "moe_route: score is sigmoid (0) or softmax (1)");
+    RoutePlan p;
+    p.n = static_cast<int>(rows * top);
+    p.top = top;
+    p.experts = static_cast<int>(experts);
+    const int tile = celeg_moe_tile_rows();
+    p.max_tiles = static_cast<int>(std::min<long long>(p.n, p.n / tile + experts));
+    const long long n = std::max(p.n, 1), tiles = std::max(p.max_tiles, 1);
+    p.ids = ws.buf("moe_ids", DType::I32, {n});
+    p.weights = ws.buf("moe_weights", DType::F32, {n});
+    p.offsets = ws.buf("moe_offsets", DType::I32, {experts + 1});
+    p.place_of = ws.buf("moe_place_of", DType::I32, {n});
+    p.entry_at = ws.buf("moe_entry_at", DType::I32, {n});
+    p.tile_expert = ws.buf("moe_tile_expert", DType::I32, {tiles});
+    p.tile_row0 = ws.buf("moe_tile_row0", DType::I32, {tiles});
+    p.n_tiles = ws.buf("moe_n_tiles", DType::I32, {4});
+    took(Path::RoutedExperts);
+    kernel_check(celeg_moe_route(logits.as<float>(), static_cast<int>(rows), p.experts, top, score, renorm ? 1 : 0,
+                                 p.ids.as<int>(), p.weights.as<float>(), stream), "moe_route");
+    kernel_check(celeg_moe_plan(p.ids.as<int>(), p.n, p.experts, p.offsets.as<int>(), p.place_of.as<int>(), p.entry_at.as<int>(),
+                                p.tile_expert.as<int>(), p.tile_row0.as<int>(), p.n_tiles.as<int>(), stream), "moe_plan");
+    return p;
+}
+
+void Ops::moe_gather(const Tensor& x, const RoutePlan& p, bool weighted, const Tensor& a) {
+    dev(x, "x");
+    dev(a, "a", x.dtype);
+    need(x.ndim == 2 && x.contiguous() && a.ndim == 2 && a.shape[0] == p.n && a.shape[1] == x.shape[1] &&
+             x.shape[0] * p.top == p.n, "moe_gather: a must be [rows * top, width]");
+    kernel_check(celeg_moe_gather(x.data, dt(x, "x"), p.entry_at.as<int>(), weighted ? p.weights.as<float>() : nullptr, a.data,
+                                  p.n, p.top, static_cast<int>(x.shape[1]), stream), "moe_gather");
+}
+
+void Ops::moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool gated, const RoutePlan& p) {
+    dev(a, "a");
+    dev(w, "w", a.dtype);
+    dev(out, "out", a.dtype);
+    need(a.ndim == 2 && w.ndim == 2 && out.ndim == 2 && a.shape[0] == p.n && out.shape[0] == p.n && w.shape[1] == a.shape[1] &&
+             w.shape[0] == static_cast<long long>(p.experts) * (gated ? 2 : 1) * out.shape[1],
+         "moe_product: a [n, K], w [experts * N (* 2 if gated), K], out [n, N]");
+    kernel_check(celeg_moe_product(a.data, w.data, out.data, dt(a, "a"), static_cast<int>(out.shape[1]),
+                                   static_cast<int>(a.shape[1]), gated ? 1 : 0, p.offsets.as<int>(), p.tile_expert.as<int>(),
+                                   p.tile_row0.as<int>(), p.n_tiles.as<int>(), p.max_tiles, stream), "moe_product");
+}
+
+void Ops::moe_combine(const Tensor& y, const RoutePlan& p, bool weighted, const Tensor& out) {
+    dev(y, "y");
+    dev(out, "out", y.dtype);
+    need(y.ndim == 2 && out.ndim == 2 && y.shape[0] == p.n && out.shape[0] * p.top == p.n && y.shape[1] == out.shape[1],
+         "moe_combine: y [rows * top, width], out [rows, width]");
+    kernel_check(celeg_moe_combine(y.data, dt(y, "y"), p.place_of.as<int>(), weighted ? p.weights.as<float>() : nullptr, out.data,
+                                   static_cast<int>(out.shape[0]), p.top, static_cast<int>(y.shape[1]), stream), "moe_combine");
 }
 
 void Ops::rmsnorm(const Tensor& x, const Tensor& weight, float eps, const Tensor& out, const Tensor* delta, const int* rows) {

@@ -102,7 +102,7 @@ struct StepPrologue {
 // graph records; a replay counts nothing): what tests and tools ask to see that a size took the
 // path it was meant to take.
 enum class Path : int {
-    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, LinearF32, LinearLibrary, LinearStandIn,
+    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, AttentionLatent, RoutedExperts, LinearF32, LinearLibrary, LinearStandIn,
     FusedSliced, FusedRows, FusedStaged, Tiled, TiledQkv, ArgmaxMerged, Count
 };
 const char* path_name(Path p);
@@ -131,7 +131,17 @@ public:
     int last_stat_blocks = 0, last_best_parts = 0, last_best_cols = 0;
 
     // row-wise
-    void embed(const Tensor& table, const int* token_ids, const Tensor& out);
+    void embed(const Tensor& table, const int* token_ids, const Tensor& out, float scale = 1.0f);
+    void scale(const Tensor& x, float factor);     // x *= factor, 32-bit x
+    // several residual streams: xs [rows, streams * width] 32-bit
+    void streams_spread(const Tensor& h, const Tensor& xs, int streams);
+    void streams_sum(const Tensor& xs, const Tensor& h, int streams);
+    // One sub-layer boundary of a row's streams: if y is given, every stream becomes
+    // sum_s mix[s, to] x_s + out_w[to] y (all from the old ones); then, if in_w is given,
+    // normed = the RMS norm (weight, eps) of sum_s in_w[s] x_s, or that sum itself in 32-bit if
+    // weight is null.
+    void hyper_step(const Tensor& xs, int streams, const Tensor* y, const Tensor* mix, const Tensor* out_w,
+                    const Tensor* in_w, const Tensor* weight, float eps, const Tensor* normed);
     void rmsnorm(const Tensor& x, const Tensor& weight, float eps, const Tensor& out, const Tensor* delta = nullptr,
                  const int* rows = nullptr);
     void swiglu(const Tensor& gate_up, const Tensor& out);
@@ -154,6 +164,36 @@ public:
     // whether a decode-only step's attention can prepare and write the step's own keys and values itself
     bool attention_fresh_ok(int heads, int head_dim, const Tensor* inv_freq, int rotary_dim, int pairing, const StepBatch& batch,
                             const KVView& kv, DType dtype) const;
+    // attention over a latent cache (one cached row per token: `rank` compressed values, then `rot`
+    // rotated key values shared by the heads)
+    struct LatentShape { int heads = 0, dim = 0, rot = 0, rank = 0; };
+    // proj [rows, ...] holds the queries [heads, dim + rot] from column q_off and (dkv) [rank + rot] from
+    // column dkv_off: the queries' rotated parts are turned in place; with `write` the normed
+    // compressed values and the turned key part go to the rows' places in the pages
+    void latent_prepare(const Tensor& proj, int q_off, int dkv_off, const LatentShape& shape, const Tensor& norm_weight,
+                        float eps, const Tensor* inv_freq, int rotary_dim, int pairing, bool write, const StepBatch& batch,
+                        const KVView& kv);
+    // out[t, h, :N] = w[h] x[t, h, :K] (w [heads, N, K]); `tail` further values of x's head pass unchanged
+    // behind them; with gate [rows, heads * N] (a view with dense rows) the result is multiplied by
+    // sigmoid(gate).  x_head / o_head: the distance between heads inside a row of x / out.
+    void headwise_linear(const Tensor& x, int x_head, const Tensor& w, const Tensor& out, int o_head, int tail,
+                         const Tensor* gate);
+    // q_lat [rows, heads * (rank + rot)] against the pages; out [rows, heads * rank]
+    void latent_attention(const Tensor& q_lat, const Tensor& out, const LatentShape& shape, float scale, const Tensor* sink,
+                          const StepBatch& batch, const KVView& kv);
+    // routed experts
+    struct RoutePlan {
+        Tensor ids, weights;                       // [rows * top]: expert and score of every (row, choice)
+        Tensor offsets, place_of, entry_at;        // rows sorted by expert
+        Tensor tile_expert, tile_row0, n_tiles;
+        int n = 0, top = 0, experts = 0, max_tiles = 0;
+    };
+    // logits [rows, experts] 32-bit -> the plan; score "sigmoid" (0) or "softmax" (1)
+    RoutePlan moe_route(const Tensor& logits, int top, int score, bool renorm, Workspace& ws);
+    void moe_gather(const Tensor& x, const RoutePlan& plan, bool weighted, const Tensor& a);
+    // out[p] = a[p] w[expert of p]^T; w [experts * N, K], or [experts * 2N, K] if gated (silu(gate) * up)
+    void moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool gated, const RoutePlan& plan);
+    void moe_combine(const Tensor& y, const RoutePlan& plan, bool weighted, const Tensor& out);
     // sampling
     void sample(const Tensor& logits, const float* fparams, const int* iparams, uint8_t* seen,
                 size_t seen_stride, int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws,

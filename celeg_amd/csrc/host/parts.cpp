@@ -1,7 +1,8 @@
 // The registries of parts and block arrangements, and the parts this library brings:
 // RMS norm, rotary and no position encoding, grouped-query attention over the paged cache,
-// the double-gated short convolution, the SwiGLU feed-forward, token embedding, tied and own
-// output head, and the pre-norm block; beside them the neutral parts ("none" mixer and
+// attention over a latent cache, the double-gated short convolution, the SwiGLU feed-forward,
+// routed experts, token embedding, tied and own output head, the pre-norm block and the block
+// on several residual streams; beside them the neutral parts ("none" mixer and
 // feed-forward, "identity" norm, "hidden" head) with which a test runs a single part alone
 // through the step function.
 #include "parts.hpp"
@@ -17,7 +18,7 @@ namespace celeg {
 namespace {
 struct Registries {
     std::map<std::string, std::map<std::string, PartFactory>> parts{
-        {"norm", {}}, {"mixer", {}}, {"ffn", {}}, {"position", {}}, {"embedding", {}}, {"head", {}}};
+        {"norm", {}}, {"mixer", {}}, {"ffn", {}}, {"position", {}}, {"embedding", {}}, {"head", {}}, {"link", {}}};
     std::map<std::string, BlockFactory> blocks;
     std::mutex lock;
 };
@@ -121,15 +122,25 @@ WeightSpec vec(long long n, const char* init = "normal") { return WeightSpec{{n}
 // RMSNorm: y = x / sqrt(mean(x^2) + eps) * w, eps inside the root, w a plain scale
 // (src/backend/cpu/kernels/elementwise.cpp:56-76; CUDA kernels/norm.cuh:1-44).  The sum of
 // squares and the scaling are done in 32-bit whatever the activation dtype.
+// "weight_offset" c: the stored weight lies around zero and the factor is c + w; the sum is
+// made once, in 32-bit, when the weight is loaded, and everything after sees a plain scale.
 class RmsNorm final : public Norm {
 public:
-    explicit RmsNorm(const PartSpec& s) : Norm(s), width_(s.params.get_int("width", 0)), eps_(s.params.get_double("eps", 0.0)) {
+    explicit RmsNorm(const PartSpec& s)
+        : Norm(s), width_(s.params.get_int("width", 0)), eps_(s.params.get_double("eps", 0.0)),
+          offset_(s.params.get_double("weight_offset", 0.0)) {
         if (width_ <= 0 || !(eps_ > 0)) throw SpecError("rmsnorm: width and eps must be positive");
     }
     bool graph_safe() const override { return true; }
-    WeightSpecs weight_specs() const override { return {{"weight", vec(width_, "around_one")}}; }
+    WeightSpecs weight_specs() const override { return {{"weight", vec(width_, offset_ != 0.0 ? "normal" : "around_one")}}; }
     void load(const PartTensors& t, Runtime&) override {
         weight_ = get(t, "weight");
+        if (offset_ != 0.0) {
+            std::vector<float> w = to_host_floats(weight_->view);
+            const float c = static_cast<float>(offset_);
+            for (float& v : w) v = c + v;
+            weight_ = from_host_floats(w, DType::F32, {width_});
+        }
         foldable_ = Foldable{weight_->view, static_cast<float>(eps_)};
     }
     void forward(const Tensor& x, const Tensor& out, Runtime& rt, const Tensor* delta, const int* rows) override {
@@ -139,7 +150,7 @@ public:
 
 private:
     long long width_;
-    double eps_;
+    double eps_, offset_;
     std::shared_ptr<DeviceTensor> weight_;
     Foldable foldable_;
 };
@@ -397,6 +408,119 @@ private:
     std::shared_ptr<DeviceTensor> w_qkv_, w_q_, w_o_, q_norm_, k_norm_;
 };
 
+// ---------------------------------------------------------------------------- latent attention
+// Attention whose keys and values are expanded from one compressed row per token.
+//
+// From the mixer's input h: q = W_q h, head by head [dim plain | rot rotated]; W_dkv h gives
+// rank + rot values: the first rank, RMS-normed with a weight of their own, are the compressed
+// row c, the last rot are a key part that every head shares and that is rotated by the
+// position, as the queries' rot part is.  Head i's key is (W_uk[i] c | shared part), its value
+// W_uv[i] c; score = (q . k) * scale over positions 0..p; softmax, whose denominator may hold
+// one more term exp(sink_i) (a learned number per head with no key and no value); the heads'
+// results, optionally times sigmoid(W_g h), go through W_o.
+//
+// Only c and the shared part are cached: one row of rank + rot values per token, in a
+// keys-only group of the cache manager.  The expansion is never made: W_uk moves to the query
+// side (q_lat[i] = (W_uk[i]^T q_plain[i] | q_rot[i]), a score is q_lat . cached row), the
+// weighted sum runs over c, and W_uv[i] is applied to it afterwards.
+class LatentAttention final : public Mixer {
+public:
+    explicit LatentAttention(const PartSpec& s) : Mixer(s) {
+        const Json& p = s.params;
+        width_ = p.get_int("width", 0);
+        shape_.heads = static_cast<int>(p.get_int("heads", 0));
+        shape_.dim = static_cast<int>(p.get_int("dim", 0));
+        shape_.rot = static_cast<int>(p.get_int("rot_dim", 0));
+        shape_.rank = static_cast<int>(p.get_int("kv_rank", 0));
+        vdim_ = static_cast<int>(p.get_int("vdim", shape_.dim));
+        eps_ = static_cast<float>(p.get_double("eps", 1e-6));
+        sink_ = p.get_bool("sink", false);
+        gate_ = p.get_bool("gate", false);
+        if (width_ <= 0 || shape_.heads <= 0 || shape_.dim <= 0 || shape_.rot < 0 || shape_.rank <= 0 || vdim_ <= 0)
+            throw SpecError("latent_attention: width, heads, dim, kv_rank and vdim must be positive");
+        scale_ = p["scale"].is_null() ? static_cast<float>(1.0 / std::sqrt(static_cast<double>(shape_.dim + shape_.rot)))
+                                      : static_cast<float>(p["scale"].as_double());
+        PartSpec none;
+        none.kind = "none";
+        position_ = build_as<PositionEncoding>(
+            "position", PartSpec::is_part(p["position"]) ? PartSpec::from_json(p["position"], "latent_attention.position") : none);
+    }
+    bool graph_safe() const override { return true; }
+    std::vector<const Part*> children() const override { return {position_.get()}; }
+    std::optional<KVNeed> kv_need() const override {
+        KVNeed need;
+        need.kv_heads = 1;
+        need.head_dim = shape_.rank + shape_.rot;
+        need.keys_only = true;
+        return need;
+    }
+    WeightSpecs weight_specs() const override {
+        const long long H = shape_.heads, qd = shape_.dim + shape_.rot;
+        WeightSpecs specs{{"q", matrix(H * qd, width_)},          {"dkv", matrix(shape_.rank + shape_.rot, width_)},
+                          {"dkv_norm", vec(shape_.rank, "around_one")}, {"uk", matrix(H * shape_.dim, shape_.rank)},
+                          {"uv", matrix(H * vdim_, shape_.rank)},  {"o", matrix(width_, H * vdim_)}};
+        if (sink_) specs.push_back({"sink", vec(H)});
+        if (gate_) specs.push_back({"g", matrix(H * vdim_, width_)});
+        return specs;
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        // q, dkv and the gate read the same rows: one product
+        std::vector<std::shared_ptr<DeviceTensor>> in{get(t, "q"), get(t, "dkv")};
+        if (gate_) in.push_back(get(t, "g"));
+        for (const auto& w : in)
+            if (w->view.dtype != in[0]->view.dtype) throw SpecError("latent_attention: the input projections are stored in different dtypes");
+        w_in_ = concat_rows(in);
+        w_o_ = get(t, "o");
+        dkv_norm_ = get(t, "dkv_norm");
+        if (sink_) sink_w_ = get(t, "sink");
+        // W_uk [heads * dim, rank] becomes [heads, rank, dim] (the query side multiplies with its transpose)
+        auto uk = get(t, "uk"), uv = get(t, "uv");
+        const int H = shape_.heads, dim = shape_.dim, rank = shape_.rank;
+        const std::vector<float> src = to_host_floats(uk->view);
+        std::vector<float> turned(src.size());
+        for (int h = 0; h < H; ++h)
+            for (int d = 0; d < dim; ++d)
+                for (int r = 0; r < rank; ++r)
+                    turned[(static_cast<size_t>(h) * rank + r) * dim + d] = src[(static_cast<size_t>(h) * dim + d) * rank + r];
+        w_uk_t_ = from_host_floats(turned, uk->view.dtype, {H, rank, dim});
+        w_uv_ = uv;
+        uv_view_ = Tensor::make(uv->view.data, uv->view.dtype, {H, vdim_, rank});
+    }
+    Tensor forward(const Tensor& x, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
+        if (!cache.kv) throw SpecError("latent_attention: the cache has no rows for this layer");
+        if (!cache.writes_kv) throw SpecError("latent_attention: reading another entry's cache is not supported");
+        const long long T = x.shape[0], H = shape_.heads;
+        const long long qd = shape_.dim + shape_.rot, D = shape_.rank + shape_.rot;
+        const long long q_cols = H * qd, dkv_cols = D, g_cols = gate_ ? H * vdim_ : 0;
+        Tensor proj = rt.ws.buf("latent_proj", rt.dtype, {T, q_cols + dkv_cols + g_cols});
+        rt.ops.linear(x, w_in_->view, proj, nullptr, rt.ws);
+        const PositionEncoding::Tables tables = position_->tables(rt);
+        const Tensor* inv_freq = tables.inv_freq.defined() ? &tables.inv_freq : nullptr;
+        rt.ops.latent_prepare(proj, 0, static_cast<int>(q_cols), shape_, dkv_norm_->view, eps_, inv_freq,
+                              inv_freq ? tables.rotary_dim : 0, tables.pairing, true, batch, *cache.kv);
+        Tensor q_lat = rt.ws.buf("latent_q", rt.dtype, {T, H * D});
+        rt.ops.headwise_linear(proj.cols(0, q_cols), static_cast<int>(qd), w_uk_t_->view, q_lat, static_cast<int>(D), shape_.rot, nullptr);
+        Tensor o_lat = rt.ws.buf("latent_o", rt.dtype, {T, H * shape_.rank});
+        rt.ops.latent_attention(q_lat, o_lat, shape_, scale_, sink_ ? &sink_w_->view : nullptr, batch, *cache.kv);
+        Tensor heads = rt.ws.buf("latent_heads", rt.dtype, {T, H * vdim_});
+        Tensor gate = gate_ ? proj.cols(q_cols + dkv_cols, g_cols) : Tensor();
+        rt.ops.headwise_linear(o_lat, shape_.rank, uv_view_, heads, vdim_, 0, gate_ ? &gate : nullptr);
+        Tensor out = rt.ws.buf("mixer_out", rt.dtype, {T, width_});
+        rt.ops.linear(heads, w_o_->view, out, nullptr, rt.ws);
+        return out;
+    }
+
+private:
+    long long width_ = 0;
+    Ops::LatentShape shape_;
+    int vdim_ = 0;
+    bool sink_ = false, gate_ = false;
+    float eps_ = 1e-6f, scale_ = 1.f;
+    std::unique_ptr<PositionEncoding> position_;
+    std::shared_ptr<DeviceTensor> w_in_, w_o_, dkv_norm_, sink_w_, w_uk_t_, w_uv_;
+    Tensor uv_view_;
+};
+
 // ---------------------------------------------------------------------------- short convolution
 // Double-gated short causal convolution.
 //
@@ -556,6 +680,76 @@ private:
     std::shared_ptr<DeviceTensor> w_gate_up_, w_down_;
 };
 
+// Routed experts: `experts` gated feed-forwards W_down (silu(W_gate x) * (W_up x)) without
+// biases, of which every row uses `top`.  Router logits z = W_router x in 32-bit (the router's
+// matrix is held in 32-bit); "score": "sigmoid" (s = 1 / (1 + e^-z), every expert by itself) or
+// "softmax" (over all experts); the `top` largest are chosen, their scores are the weights
+// ("renormalize": divided by their sum).  "weight_on": "input" (the output is
+// sum expert(w x)) or "output" (sum w expert(x)).
+class RoutedExperts final : public FeedForward {
+public:
+    explicit RoutedExperts(const PartSpec& s) : FeedForward(s) {
+        const Json& p = s.params;
+        width_ = p.get_int("width", 0);
+        ff_ = p.get_int("ff", 0);
+        experts_ = static_cast<int>(p.get_int("experts", 0));
+        top_ = static_cast<int>(p.get_int("top", 0));
+        const std::string score = p.get_string("score", "sigmoid"), on = p.get_string("weight_on", "output");
+        if (score != "sigmoid" && score != "softmax") throw SpecError("routed_experts: score is 'sigmoid' or 'softmax', not '" + score + "'");
+        if (on != "input" && on != "output") throw SpecError("routed_experts: weight_on is 'input' or 'output', not '" + on + "'");
+        score_ = score == "softmax" ? 1 : 0;
+        on_input_ = on == "input";
+        renorm_ = p.get_bool("renormalize", false);
+        if (width_ <= 0 || ff_ <= 0 || experts_ <= 0 || top_ <= 0 || top_ > experts_)
+            throw SpecError("routed_experts: width, ff and experts must be positive and top between 1 and experts");
+    }
+    bool graph_safe() const override { return true; }
+    static std::string role(const char* what, int e) { return std::string(what) + "." + std::to_string(e); }
+    WeightSpecs weight_specs() const override {
+        WeightSpecs specs{{"router", WeightSpec{{experts_, width_}, "vector", "normal", {}}}};
+        for (int e = 0; e < experts_; ++e) {
+            specs.push_back({role("gate", e), matrix(ff_, width_)});
+            specs.push_back({role("up", e), matrix(ff_, width_)});
+            specs.push_back({role("down", e), matrix(width_, ff_)});
+        }
+        return specs;
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        router_ = get(t, "router");
+        std::vector<std::shared_ptr<DeviceTensor>> in, out;
+        for (int e = 0; e < experts_; ++e) {
+            in.push_back(get(t, role("gate", e)));
+            in.push_back(get(t, role("up", e)));
+            out.push_back(get(t, role("down", e)));
+        }
+        for (const auto& w : in)
+            if (w->view.dtype != in[0]->view.dtype) throw SpecError("routed_experts: the experts are stored in different dtypes");
+        w_gate_up_ = concat_rows(in);       // [experts * 2 ff, width]: per expert its gate rows, then its up rows
+        w_down_ = concat_rows(out);         // [experts * width, ff]
+    }
+    Tensor forward(const Tensor& x, const StepBatch&, Runtime& rt) override {
+        const long long T = x.shape[0];
+        Tensor logits = rt.ws.buf("moe_logits", DType::F32, {T, experts_});
+        rt.ops.linear(x, router_->view, logits, nullptr, rt.ws);
+        const Ops::RoutePlan plan = rt.ops.moe_route(logits, top_, score_, renorm_, rt.ws);
+        Tensor a = rt.ws.buf("moe_in", rt.dtype, {T * top_, width_});
+        rt.ops.moe_gather(x, plan, on_input_, a);
+        Tensor act = rt.ws.buf("moe_act", rt.dtype, {T * top_, ff_});
+        rt.ops.moe_product(a, w_gate_up_->view, act, true, plan);
+        Tensor y = rt.ws.buf("moe_y", rt.dtype, {T * top_, width_});
+        rt.ops.moe_product(act, w_down_->view, y, false, plan);
+        Tensor out = rt.ws.buf("ffn_out", rt.dtype, {T, width_});
+        rt.ops.moe_combine(y, plan, !on_input_, out);
+        return out;
+    }
+
+private:
+    long long width_ = 0, ff_ = 0;
+    int experts_ = 0, top_ = 0, score_ = 0;
+    bool on_input_ = false, renorm_ = false;
+    std::shared_ptr<DeviceTensor> router_, w_gate_up_, w_down_;
+};
+
 // a layer without a feed-forward (the reference's LayerSpec may hold none,
 // src/model/inference/rules.cpp:44-46)
 class NoFeedForward final : public FeedForward {
@@ -569,10 +763,13 @@ public:
 // h0[t] = E[token[t]], nothing added and no scaling (src/backend/cpu/model_forward_token.cpp:28-60);
 // logits = x E_out^T with E_out = E when the head is tied, else lm_head
 // (src/backend/cpu/model_forward_token.cpp:213-218; src/model/inference/layer_bindings.cpp:24-95).
-// Logits leave in 32-bit.
+// Logits leave in 32-bit.  "scale" on the embedding multiplies the gathered rows (in 32-bit, as
+// they enter the residual stream); "scale" on a head multiplies the logits.
 class TokenEmbedding final : public Embedding {
 public:
-    explicit TokenEmbedding(const PartSpec& s) : Embedding(s), vocab_(s.params.get_int("vocab", 0)), width_(s.params.get_int("width", 0)) {
+    explicit TokenEmbedding(const PartSpec& s)
+        : Embedding(s), vocab_(s.params.get_int("vocab", 0)), width_(s.params.get_int("width", 0)),
+          scale_(static_cast<float>(s.params.get_double("scale", 1.0))) {
         if (vocab_ <= 0 || width_ <= 0) throw SpecError("embedding: vocab and width must be positive");
     }
     bool graph_safe() const override { return true; }
@@ -582,6 +779,13 @@ public:
     bool takes_step_prologue() const override { return true; }
     void forward(const int* token_ids, const Tensor& out, Runtime& rt, const StepBatch* batch) override {
         const int rows = static_cast<int>(out.shape[0]);
+        if (scale_ != 1.0f) {
+            rt.flush_prologue();
+            rt.ops.embed(table_->view, token_ids, out, scale_);
+            rt.stream_stat_blocks = 0;
+            rt.stream_has_bf16 = false;
+            return;
+        }
         if (batch && table_->view.dtype == DType::BF16 && fused::fused_rows_ok(rt, *batch, {width_})) {
             // few rows: leave every row's sum of squares (and the bfloat16 copy of the stream)
             // for the first norm
@@ -607,6 +811,7 @@ public:
 
 private:
     long long vocab_, width_;
+    float scale_;
     std::shared_ptr<DeviceTensor> table_;
 };
 
@@ -643,14 +848,17 @@ bool head_fused(const Tensor& h, const Norm::Foldable& norm, const StepBatch& ba
 // uses the embedding table; wants no tensor of its own
 class TiedHead final : public Head {
 public:
-    explicit TiedHead(const PartSpec& s) : Head(s), vocab_(static_cast<int>(s.params.get_int("vocab", 0))) {}
+    explicit TiedHead(const PartSpec& s)
+        : Head(s), vocab_(static_cast<int>(s.params.get_int("vocab", 0))), scale_(static_cast<float>(s.params.get_double("scale", 1.0))) {}
     bool graph_safe() const override { return true; }
     int vocab() const override { return vocab_; }
     void forward(const Tensor& x, const Tensor& out, Runtime& rt, const Embedding* embedding) override {
         rt.ops.linear(x, table_of(embedding), out, nullptr, rt.ws);
+        if (scale_ != 1.0f) rt.ops.scale(out, scale_);
     }
     bool forward_fused(const Tensor& h, const Norm::Foldable& norm, const StepBatch& batch, const Tensor& out, Runtime& rt,
                        const Embedding* embedding) override {
+        if (scale_ != 1.0f) return false;       // (what the fused head leaves beside the logits knows no scale)
         return head_fused(h, norm, batch, out, rt, table_of(embedding));
     }
 
@@ -661,27 +869,32 @@ private:
         return t;
     }
     int vocab_;
+    float scale_;
 };
 
 class LinearHead final : public Head {
 public:
     explicit LinearHead(const PartSpec& s)
-        : Head(s), vocab_(static_cast<int>(s.params.get_int("vocab", 0))), width_(s.params.get_int("width", 0)) {}
+        : Head(s), vocab_(static_cast<int>(s.params.get_int("vocab", 0))), width_(s.params.get_int("width", 0)),
+          scale_(static_cast<float>(s.params.get_double("scale", 1.0))) {}
     bool graph_safe() const override { return true; }
     int vocab() const override { return vocab_; }
     WeightSpecs weight_specs() const override { return {{"weight", matrix(vocab_, width_)}}; }
     void load(const PartTensors& t, Runtime&) override { weight_ = get(t, "weight"); }
     void forward(const Tensor& x, const Tensor& out, Runtime& rt, const Embedding*) override {
         rt.ops.linear(x, weight_->view, out, nullptr, rt.ws);
+        if (scale_ != 1.0f) rt.ops.scale(out, scale_);
     }
     bool forward_fused(const Tensor& h, const Norm::Foldable& norm, const StepBatch& batch, const Tensor& out, Runtime& rt,
                        const Embedding*) override {
+        if (scale_ != 1.0f) return false;
         return head_fused(h, norm, batch, out, rt, weight_->view);
     }
 
 private:
     int vocab_;
     long long width_;
+    float scale_;
     std::shared_ptr<DeviceTensor> weight_;
 };
 
@@ -747,6 +960,104 @@ private:
     std::unique_ptr<FeedForward> ffn_;
 };
 
+// ---------------------------------------------------------------------------- several residual streams
+// How one sub-layer hangs on a row's S residual streams: it reads sum_s in[s] x_s, and its
+// output y comes back as x_t <- sum_s mix[s, t] x_s + out[t] y (mix indexed [from, to]).
+class HyperLink final : public Part {
+public:
+    explicit HyperLink(const PartSpec& s) : Part(s), streams_(static_cast<int>(s.params.get_int("streams", 0))) {
+        if (streams_ <= 0 || streams_ > 8) throw SpecError("hyper_link: between 1 and 8 streams");
+    }
+    bool graph_safe() const override { return true; }
+    WeightSpecs weight_specs() const override {
+        return {{"in", vec(streams_, "around_one")}, {"out", vec(streams_, "around_one")},
+                {"mix", WeightSpec{{streams_, streams_}, "vector", "around_one", {}}}};
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        in = get(t, "in");
+        out = get(t, "out");
+        mix = get(t, "mix");
+    }
+    int streams() const { return streams_; }
+    std::shared_ptr<DeviceTensor> in, out, mix;
+
+private:
+    int streams_;
+};
+
+// hyper_connections: the pre-norm order of work on S streams h [T, S * width].  A kernel at each
+// sub-layer boundary writes the previous output back into the streams, mixes the next input and
+// normalises it.  A sub-layer of kind "none" is left out altogether.
+class HyperBlock final : public Block {
+public:
+    explicit HyperBlock(const LayerSpec& layer)
+        : mixer_norm_(build_as<Norm>("norm", layer.mixer_norm)), mixer_(build_as<Mixer>("mixer", layer.mixer)),
+          mixer_link_(build_as<HyperLink>("link", layer.mixer_link)), has_ffn_(layer.ffn.kind != "none") {
+        if (has_ffn_) {
+            ffn_norm_ = build_as<Norm>("norm", layer.ffn_norm);
+            ffn_ = build_as<FeedForward>("ffn", layer.ffn);
+            ffn_link_ = build_as<HyperLink>("link", layer.ffn_link);
+            if (ffn_link_->streams() != mixer_link_->streams()) throw SpecError("hyper_connections: the links of a layer differ in streams");
+        }
+    }
+    std::vector<std::pair<std::string, Part*>> parts() override {
+        std::vector<std::pair<std::string, Part*>> out{{"mixer_norm", mixer_norm_.get()}, {"mixer", mixer_.get()}, {"mixer_link", mixer_link_.get()}};
+        if (has_ffn_) {
+            out.emplace_back("ffn_norm", ffn_norm_.get());
+            out.emplace_back("ffn", ffn_.get());
+            out.emplace_back("ffn_link", ffn_link_.get());
+        }
+        return out;
+    }
+    Mixer& mixer() override { return *mixer_; }
+    int streams() const override { return mixer_link_->streams(); }
+    Tensor forward(const Tensor& h, const Tensor& delta, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
+        const int S = streams();
+        if (delta.defined()) throw SpecError("hyper_connections: a pending addition from a block of another arrangement");
+        if (h.shape[1] % S) throw SpecError("hyper_connections: the rows do not hold a whole number of streams");
+        const long long T = h.shape[0], width = h.shape[1] / S;
+        rt.stream_stat_blocks = 0;
+        rt.stream_has_bf16 = false;
+        Tensor normed = rt.ws.buf("normed", rt.dtype, {T, width});
+        read(h, S, nullptr, nullptr, *mixer_link_, *mixer_norm_, normed, rt);
+        Tensor y = mixer_->forward(normed, batch, cache, rt);
+        rt.mark("mixer " + mixer_->spec.kind);
+        const HyperLink* pending = mixer_link_.get();
+        if (has_ffn_) {
+            read(h, S, &y, pending, *ffn_link_, *ffn_norm_, normed, rt);
+            y = ffn_->forward(normed, batch, rt);
+            rt.mark("ffn " + ffn_->spec.kind);
+            pending = ffn_link_.get();
+        }
+        rt.ops.hyper_step(h, S, &y, &pending->mix->view, &pending->out->view, nullptr, nullptr, 0.f, nullptr);
+        return Tensor();
+    }
+
+private:
+    // writes y back through `from` (if given), then normed = norm(sum_s in[s] x_s)
+    static void read(const Tensor& h, int S, const Tensor* y, const HyperLink* from, const HyperLink& to, Norm& norm,
+                     const Tensor& normed, Runtime& rt) {
+        const Norm::Foldable* fold = norm.foldable();
+        const Tensor* mix = from ? &from->mix->view : nullptr;
+        const Tensor* out = from ? &from->out->view : nullptr;
+        if (fold) {
+            rt.ops.hyper_step(h, S, y, mix, out, &to.in->view, &fold->weight, fold->eps, &normed);
+            return;
+        }
+        // a norm that is not an RMS norm: the mixture leaves in 32-bit and the norm runs by itself
+        Tensor u = rt.ws.buf("hyper_mixture", DType::F32, {normed.shape[0], normed.shape[1]});
+        rt.ops.hyper_step(h, S, y, mix, out, &to.in->view, nullptr, 0.f, &u);
+        norm.forward(u, normed, rt, nullptr, nullptr);
+    }
+    std::unique_ptr<Norm> mixer_norm_;
+    std::unique_ptr<Mixer> mixer_;
+    std::unique_ptr<HyperLink> mixer_link_;
+    bool has_ffn_;
+    std::unique_ptr<Norm> ffn_norm_;
+    std::unique_ptr<FeedForward> ffn_;
+    std::unique_ptr<HyperLink> ffn_link_;
+};
+
 template <typename T>
 PartFactory factory_of() {
     return [](const PartSpec& s) { return std::unique_ptr<Part>(new T(s)); };
@@ -760,15 +1071,19 @@ void register_builtin_parts() {
     r.parts["position"]["rope"] = factory_of<Rope>();
     r.parts["position"]["none"] = factory_of<NoPosition>();
     r.parts["mixer"]["gqa_attention"] = factory_of<GqaAttention>();
+    r.parts["mixer"]["latent_attention"] = factory_of<LatentAttention>();
     r.parts["mixer"]["short_conv"] = factory_of<ShortConv>();
     r.parts["mixer"]["none"] = factory_of<NoMixer>();
     r.parts["ffn"]["swiglu"] = factory_of<SwiGlu>();
+    r.parts["ffn"]["routed_experts"] = factory_of<RoutedExperts>();
     r.parts["ffn"]["none"] = factory_of<NoFeedForward>();
+    r.parts["link"]["hyper_link"] = factory_of<HyperLink>();
     r.parts["embedding"]["embedding"] = factory_of<TokenEmbedding>();
     r.parts["head"]["tied_head"] = factory_of<TiedHead>();
     r.parts["head"]["linear_head"] = factory_of<LinearHead>();
     r.parts["head"]["hidden"] = factory_of<HiddenHead>();
     r.blocks["pre_norm"] = [](const LayerSpec& layer) { return std::unique_ptr<Block>(new PreNormBlock(layer)); };
+    r.blocks["hyper_connections"] = [](const LayerSpec& layer) { return std::unique_ptr<Block>(new HyperBlock(layer)); };
 }
 
 }  // namespace

@@ -123,6 +123,8 @@ public:
     virtual ~Block() = default;
     virtual std::vector<std::pair<std::string, Part*>> parts() = 0;
     virtual Mixer& mixer() = 0;
+    // residual streams a row of h holds for this block: h is [T, streams * width]
+    virtual int streams() const { return 1; }
     virtual Tensor forward(const Tensor& h, const Tensor& delta, const StepBatch& batch, const LayerCache& cache, Runtime& rt) = 0;
 };
 
@@ -130,7 +132,7 @@ public:
 using PartFactory = std::function<std::unique_ptr<Part>(const PartSpec&)>;
 using BlockFactory = std::function<std::unique_ptr<Block>(const LayerSpec&)>;
 
-// role: norm, mixer, ffn, position, embedding, head
+// role: norm, mixer, ffn, position, embedding, head, link
 void register_part(const std::string& role, const std::string& kind, PartFactory factory, bool replace = false);
 void register_block(const std::string& arrangement, BlockFactory factory, bool replace = false);
 std::unique_ptr<Part> build_part(const std::string& role, const PartSpec& spec);

@@ -12,8 +12,10 @@
 //   part:  {"kind": .., "params": {..}, "tensors": {role: checkpoint name}}; a parameter
 //          may itself be a part (an attention's "position")
 //   layer: {"mixer": part, "mixer_norm": part, "ffn": part, "ffn_norm": part,
-//           "arrangement": "pre_norm"}
-//   model: {"architecture", "vocab_size", "hidden_size", "max_context", "embedding": part,
+//           "arrangement": "pre_norm"}; an arrangement that joins a sub-layer to the residual
+//           stream by a part of its own names them as "mixer_link" and "ffn_link"
+//   model: {"architecture", "vocab_size", "hidden_size", "max_context", "streams" (residual
+//           streams per row, 1 if absent), "embedding": part,
 //           "layers": [layer], "order": [{"layer": i, "kv_from": j or null}],
 //           "final_norm": part, "head": part, "eos_token_ids": [..], "bos_token_id"}
 #pragma once
@@ -74,6 +76,9 @@ struct PartSpec {
 
 struct LayerSpec {
     PartSpec mixer, mixer_norm, ffn, ffn_norm;
+    // how each sub-layer reads from and writes to the residual stream(s), for arrangements in
+    // which that is a part with weights of its own (kind empty: the arrangement has none)
+    PartSpec mixer_link, ffn_link;
     std::string arrangement = "pre_norm";
 };
 
@@ -89,6 +94,7 @@ struct RunStep {
 struct ModelSpec {
     std::string architecture;
     int vocab_size = 0, hidden_size = 0, max_context = 0;
+    int streams = 1;             // residual streams a row keeps between layers
     PartSpec embedding;
     std::vector<LayerSpec> layers;
     std::vector<RunStep> order;
@@ -99,6 +105,7 @@ struct ModelSpec {
     void validate() const {
         if (vocab_size <= 0 || hidden_size <= 0 || max_context <= 0)
             throw SpecError("vocab_size, hidden_size and max_context must be positive");
+        if (streams <= 0) throw SpecError("streams must be positive");
         if (order.empty()) throw SpecError("the run order is empty");
         for (size_t i = 0; i < order.size(); ++i) {
             if (order[i].layer < 0 || order[i].layer >= static_cast<int>(layers.size()))
@@ -113,15 +120,19 @@ struct ModelSpec {
 
     Json to_json() const {
         Json ls = Json::array();
-        for (const auto& l : layers)
-            ls.push(Json::object().set("mixer", l.mixer.to_json()).set("mixer_norm", l.mixer_norm.to_json())
-                        .set("ffn", l.ffn.to_json()).set("ffn_norm", l.ffn_norm.to_json())
-                        .set("arrangement", l.arrangement));
+        for (const auto& l : layers) {
+            Json lj = Json::object().set("mixer", l.mixer.to_json()).set("mixer_norm", l.mixer_norm.to_json())
+                          .set("ffn", l.ffn.to_json()).set("ffn_norm", l.ffn_norm.to_json())
+                          .set("arrangement", l.arrangement);
+            if (!l.mixer_link.kind.empty()) lj.set("mixer_link", l.mixer_link.to_json());
+            if (!l.ffn_link.kind.empty()) lj.set("ffn_link", l.ffn_link.to_json());
+            ls.push(lj);
+        }
         Json ord = Json::array();
         for (const auto& s : order)
             ord.push(Json::object().set("layer", s.layer).set("kv_from", s.kv_from ? Json(*s.kv_from) : Json()));
         return Json::object().set("architecture", architecture).set("vocab_size", vocab_size)
-            .set("hidden_size", hidden_size).set("max_context", max_context)
+            .set("hidden_size", hidden_size).set("max_context", max_context).set("streams", streams)
             .set("embedding", embedding.to_json()).set("layers", ls).set("order", ord)
             .set("final_norm", final_norm.to_json()).set("head", head.to_json())
             .set("eos_token_ids", Json::array_of(eos_token_ids))
@@ -135,6 +146,7 @@ struct ModelSpec {
         m.vocab_size = static_cast<int>(j.get_int("vocab_size", 0));
         m.hidden_size = static_cast<int>(j.get_int("hidden_size", 0));
         m.max_context = static_cast<int>(j.get_int("max_context", 0));
+        m.streams = static_cast<int>(j.get_int("streams", 1));
         m.embedding = PartSpec::from_json(j["embedding"], "embedding");
         if (!j["layers"].is_array()) throw SpecError("\"layers\" must be an array");
         int n = 0;
@@ -145,6 +157,8 @@ struct ModelSpec {
             ls.mixer_norm = PartSpec::from_json(l["mixer_norm"], where + ".mixer_norm");
             ls.ffn = PartSpec::from_json(l["ffn"], where + ".ffn");
             ls.ffn_norm = PartSpec::from_json(l["ffn_norm"], where + ".ffn_norm");
+            if (!l["mixer_link"].is_null()) ls.mixer_link = PartSpec::from_json(l["mixer_link"], where + ".mixer_link");
+            if (!l["ffn_link"].is_null()) ls.ffn_link = PartSpec::from_json(l["ffn_link"], where + ".ffn_link");
             ls.arrangement = l.get_string("arrangement", "pre_norm");
             m.layers.push_back(std::move(ls));
         }
