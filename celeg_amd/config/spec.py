@@ -39,11 +39,27 @@ class LayerSpec:
     ffn: PartSpec
     ffn_norm: PartSpec
     arrangement: str = "pre_norm"
+    # how each sub-layer hangs on the residual stream(s), where the arrangement makes that a
+    # part with weights of its own ("hyper_connections": a "hyper_link" each)
+    mixer_link: Optional[PartSpec] = None
+    ffn_link: Optional[PartSpec] = None
 
     def to_json(self) -> Dict[str, Any]:
-        return {"mixer": self.mixer.to_json(), "mixer_norm": self.mixer_norm.to_json(),
-                "ffn": self.ffn.to_json(), "ffn_norm": self.ffn_norm.to_json(),
-                "arrangement": self.arrangement}
+        out = {"mixer": self.mixer.to_json(), "mixer_norm": self.mixer_norm.to_json(),
+               "ffn": self.ffn.to_json(), "ffn_norm": self.ffn_norm.to_json(),
+               "arrangement": self.arrangement}
+        if self.mixer_link is not None:
+            out["mixer_link"] = self.mixer_link.to_json()
+        if self.ffn_link is not None:
+            out["ffn_link"] = self.ffn_link.to_json()
+        return out
+
+    @classmethod
+    def from_json(cls, l: Dict[str, Any]) -> "LayerSpec":
+        link = lambda key: PartSpec.from_json(l[key]) if l.get(key) else None
+        return cls(PartSpec.from_json(l["mixer"]), PartSpec.from_json(l["mixer_norm"]),
+                   PartSpec.from_json(l["ffn"]), PartSpec.from_json(l["ffn_norm"]),
+                   l.get("arrangement", "pre_norm"), link("mixer_link"), link("ffn_link"))
 
 
 @dataclass(frozen=True)
@@ -69,10 +85,11 @@ class ModelSpec:
     head: PartSpec
     eos_token_ids: Tuple[int, ...] = ()
     bos_token_id: Optional[int] = None
+    streams: int = 1          # residual streams a row keeps between layers
 
     def to_json(self) -> Dict[str, Any]:
         return {"architecture": self.architecture, "vocab_size": self.vocab_size,
-                "hidden_size": self.hidden_size, "max_context": self.max_context,
+                "hidden_size": self.hidden_size, "max_context": self.max_context, "streams": self.streams,
                 "embedding": self.embedding.to_json(), "layers": [l.to_json() for l in self.layers],
                 "order": [{"layer": s.layer, "kv_from": s.kv_from} for s in self.order],
                 "final_norm": self.final_norm.to_json(), "head": self.head.to_json(),
@@ -80,13 +97,12 @@ class ModelSpec:
 
     @classmethod
     def from_json(cls, j: Dict[str, Any]) -> "ModelSpec":
-        layers = tuple(LayerSpec(PartSpec.from_json(l["mixer"]), PartSpec.from_json(l["mixer_norm"]),
-                                 PartSpec.from_json(l["ffn"]), PartSpec.from_json(l["ffn_norm"]),
-                                 l.get("arrangement", "pre_norm")) for l in j["layers"])
+        layers = tuple(LayerSpec.from_json(l) for l in j["layers"])
         order = tuple(RunStep(s["layer"], s.get("kv_from")) for s in j["order"])
         return cls(j["architecture"], j["vocab_size"], j["hidden_size"], j["max_context"],
                    PartSpec.from_json(j["embedding"]), layers, order, PartSpec.from_json(j["final_norm"]),
-                   PartSpec.from_json(j["head"]), tuple(j.get("eos_token_ids") or ()), j.get("bos_token_id"))
+                   PartSpec.from_json(j["head"]), tuple(j.get("eos_token_ids") or ()), j.get("bos_token_id"),
+                   int(j.get("streams") or 1))
 
     def tensor_names(self) -> List[str]:
         names: List[str] = []
@@ -98,5 +114,6 @@ class ModelSpec:
         parts = [self.embedding]
         for layer in self.layers:
             parts += [layer.mixer_norm, layer.mixer, layer.ffn_norm, layer.ffn]
+            parts += [p for p in (layer.mixer_link, layer.ffn_link) if p is not None]
         parts += [self.final_norm, self.head]
         return parts

@@ -971,7 +971,7 @@ public:
     bool graph_safe() const override { return true; }
     WeightSpecs weight_specs() const override {
         return {{"in", vec(streams_, "around_one")}, {"out", vec(streams_, "around_one")},
-                {"mix", WeightSpec{{streams_, streams_}, "vector", "around_one", {}}}};
+                {"mix", WeightSpec{{streams_, streams_}, "vector", "around_identity", {}}}};
     }
     void load(const PartTensors& t, Runtime&) override {
         in = get(t, "in");

@@ -5,7 +5,8 @@ The reference has no such mode (its tests use shapes only,
 tests/automatic_inference_test.cpp:13-38).  Every tensor is drawn from a generator
 keyed by (seed, tensor name), so a tensor's values do not depend on which other
 tensors exist or on the order of writing: matrices, tables, biases and filter taps
-are N(0, std); norm scales are 1 + N(0, std).  Values are drawn in 32-bit and then
+are N(0, std); norm scales are 1 + N(0, std) (N(0, std) where the factor is 1 + w); a
+matrix that mixes residual streams is the identity + N(0, std).  Values are drawn in 32-bit and then
 rounded to the storage dtype.
 """
 from __future__ import annotations
@@ -32,6 +33,8 @@ def random_tensor(seed: int, name: str, shape, init: str, std: float) -> torch.T
     t = torch.randn(tuple(shape), generator=tensor_generator(seed, name), dtype=torch.float32) * std
     if init == "around_one":
         t = t + 1.0
+    elif init == "around_identity":
+        t = t + torch.eye(int(shape[0]), int(shape[1]))
     elif init != "normal":
         raise ValueError(f"unknown initialisation '{init}'")
     return t
