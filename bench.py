@@ -126,6 +126,69 @@ def serve(shape: str, chunk: int = 0, budget: int = 0, granule: int = 1, gemm_ba
     return 0
 
 
+# Regipel at sizes that resemble a real model's layers, each beside the closest existing model at
+# equal size: an LFM2 shape of attention layers only, with the same width, layers, heads and
+# vocabulary, and a dense feed-forward as wide as the experts a token uses together.
+def regipel_shape(width, layers, heads, dim, rot, vdim, rank, experts, top, ff, streams=2, vocab=65536):
+    mixer = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "scale": (dim + rot) ** -0.5,
+             "rot": {"base": 500000.0, "dims": rot}}
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    return {"architecture": "Regipel", "vocab": vocab, "width": width, "streams": streams, "norm": {"eps": 1e-5},
+            "embedding": {"scale": float(width) ** 0.5}, "logit_scale": 0.5, "max_context": 8192,
+            "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": mlp} for _ in range(layers)]}
+
+
+DESIGN_SHAPES = {
+    "1k": (regipel_shape(1024, 8, 16, 64, 32, 64, 256, 16, 2, 1024), lfm2_shape(1024, 16, 8, 2048, set(range(8)), 8, 8192)),
+    "2k": (regipel_shape(2048, 8, 16, 128, 64, 128, 512, 32, 4, 1024), lfm2_shape(2048, 32, 8, 4096, set(range(8)), 8, 8192)),
+}
+
+
+def design(shapes, steps: int, warmup: int, batch: int, layers: int = 0, profile_only: str = "") -> int:
+    """Prefill of 2,048 tokens and decode at `batch` requests of 2,048 tokens, for every shape and
+    both models.  Prints one JSON line."""
+    import torch
+    from celeg_amd.engine import Engine
+    from celeg_amd.engine.benchmark import DecodeBench, measure_prefill
+    from celeg_amd.weights import write_random_model
+    out = {}
+    for shape in shapes:
+        for label, cfg in zip(("regipel", "lfm2_attention"), DESIGN_SHAPES[shape]):
+            if profile_only and label != profile_only:
+                continue
+            cfg = json.loads(json.dumps(cfg))
+            if layers:
+                if label == "regipel":
+                    cfg["layers"] = cfg["layers"][:layers]
+                else:
+                    cfg.update(num_hidden_layers=layers, layer_types=cfg["layer_types"][:layers])
+            cfg.pop("block_auto_adjust_ff_dim", None)
+            need = PROMPT_TOKENS + steps + warmup + batch + 3
+            with tempfile.TemporaryDirectory(prefix="celeg_bench_") as folder:
+                write_random_model(cfg, folder, seed=0, dtype=torch.bfloat16, std=0.02)
+                engine = Engine.from_folder(folder, dtype="bfloat16", device="cuda:0", page_tokens=16,
+                                            n_pages=((need + 15) // 16 + 1) * batch, max_active_requests=batch,
+                                            context=need + 16, max_batched_tokens=PROMPT_TOKENS,
+                                            prefill_chunk_tokens=PROMPT_TOKENS)
+            lm = engine.loaded
+            prefill = measure_prefill(lm, PROMPT_TOKENS, repeats=5, warmup=2)
+            bench = DecodeBench(engine, batch, PROMPT_TOKENS, steps + warmup + batch + 2, seed=batch)
+            decode = bench.run(steps, warmup)
+            bench.close()
+            out[f"{shape}/{label}"] = {
+                "prefill_tokens_per_second": round(prefill["tokens_per_second"], 1), "prefill_ms": round(prefill["ms"], 3),
+                "decode_tokens_per_second": round(decode["tokens_per_second"], 1),
+                "decode_ms_per_step": round(decode["ms_per_step"], 4),
+                "weights": lm.native.info["weights"], "kv_bytes_per_token": lm.native.info["kv_bytes_per_token"],
+                "layers": len(lm.native.info["spec"]["order"])}
+            engine.close()
+    print(json.dumps({"metric": "Regipel beside LFM2 attention layers at equal size: prefill tok/s @ 2048 tokens, "
+                                f"decode tok/s @ batch {batch}, context 2048 (bf16, random weights)",
+                      "phase": "design", "batch": batch, "steps": steps, "warmup": warmup, "dtype": "bf16",
+                      "data": "synthetic", "shapes": out}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -147,10 +210,14 @@ def main() -> int:
                     help="with --phase decode: tokens every request holds when decoding starts "
                          "(default 2048, the headline's); with --phase prefill: tokens of the same "
                          "prompt that the cache holds before the measured portion of 2,048 (default 0)")
-    ap.add_argument("--phase", choices=["all", "prefill", "decode", "serve"], default="all",
+    ap.add_argument("--design-shape", default="1k,2k", help="with --phase design: which sizes (1k, 2k)")
+    ap.add_argument("--design-model", default="", choices=["", "regipel", "lfm2_attention"],
+                    help="with --phase design: only this model (for profiling)")
+    ap.add_argument("--phase", choices=["all", "prefill", "decode", "serve", "design"], default="all",
                     help="for profiling: run only the prefill measurement, or only the batch-8 "
                          "decode measurement (the line printed then holds only that part); "
-                         "serve: the whole engine on the serving workload of --shape")
+                         "serve: the whole engine on the serving workload of --shape; design: the "
+                         "Regipel design beside LFM2 attention layers at equal size")
     ap.add_argument("--knob", action="append", default=[], metavar="NAME=VALUE",
                     help="set a knob of the step function or the kernels' dispatch before measuring "
                          "(tuning runs; the names are those of celeg_model_knobs)")
@@ -162,6 +229,9 @@ def main() -> int:
               "(this engine runs on a single MI355X)")
         return 2
 
+    if args.phase == "design":
+        return design(args.design_shape.split(","), min(args.steps, 64), min(args.warmup, 8), args.batch, args.layers,
+                      args.design_model)
     if args.phase == "serve":
         return serve(args.shape, args.prefill_chunk, args.token_budget, args.portion_granule, args.gemm_backend)
 

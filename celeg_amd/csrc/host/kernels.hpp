@@ -44,6 +44,13 @@ int celeg_latent_attention(const void* q, int ldq, const void* pool, int dtype, 
                            const int* token_slot, const int* positions, const float* sink, void* out, int ldo,
                            int n_tokens, int heads, int rank, int rot, int page_tokens, int n_layers, int layer,
                            float scale, hipStream_t stream);
+// latent_fast.hip
+int celeg_latent_attention_fast_ok(int rank, int rot);
+int celeg_latent_attention_fast(int form, const void* q, int ldq, const void* pool, const int* table, int table_stride,
+                                const int* cu_seqlens, const int* seq_slot, const int* seq_start, int n_seqs, int max_tiles,
+                                const int* token_slot, const int* positions, int n_single, const float* sink, void* out,
+                                int ldo, float* ws_o, float* ws_ml, int n_splits, int blocks_per_split, int heads, int rank,
+                                int rot, int page_tokens, int n_layers, int layer, float scale, hipStream_t stream);
 // moe.hip
 int celeg_moe_route(const float* logits, int rows, int experts, int top, int score, int renorm, int* ids, float* weights,
                     hipStream_t stream);

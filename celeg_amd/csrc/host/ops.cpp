@@ -52,6 +52,8 @@ const char* path_name(Path p) {
         case Path::AttentionRows: return "attention_rows";
         case Path::AttentionGeneral: return "attention_general";
         case Path::AttentionLatent: return "attention_latent";
+        case Path::AttentionLatentRows: return "attention_latent_rows";
+        case Path::AttentionLatentDecode: return "attention_latent_decode";
         case Path::RoutedExperts: return "routed_experts";
         case Path::LinearF32: return "linear_f32";
         case Path::LinearLibrary: return "linear_library";
@@ -202,7 +204,7 @@ void Ops::headwise_linear(const Tensor& x, int x_head, const Tensor& w, const Te
 }
 
 void Ops::latent_attention(const Tensor& q_lat, const Tensor& out, const LatentShape& s, float scale, const Tensor* sink,
-                           const StepBatch& batch, const KVView& kv) {
+                           const StepBatch& batch, const KVView& kv, Workspace& ws) {
     dev(q_lat, "q_lat");
     dev(out, "out", q_lat.dtype);
     const int D = s.rank + s.rot;
@@ -217,6 +219,40 @@ void Ops::latent_attention(const Tensor& q_lat, const Tensor& out, const LatentS
     }
     latent_cache_fits(s, kv, q_lat.dtype, "latent_attention");
     took(Path::AttentionLatent);
+    if (q_lat.dtype == DType::BF16 && use_latent_mfma && !attention_general && scale > 0.f && out.contiguous() &&
+        celeg_latent_attention_fast_ok(s.rank, s.rot)) {
+        const int T = batch.n_tokens, n_single = std::min(batch.single_rows, T);
+        const float* sink_p = sink ? sink->as<float>() : nullptr;
+        if (n_single > 0) {
+            // single tokens: the keys of a row in shares, so that the chip is busy whatever the batch
+            const int blocks = (std::max(hint_of(batch, kv), 1) + 63) / 64;
+            const int groups = n_single * ((s.heads + 15) / 16);
+            int n_splits = std::clamp(latent_decode_workgroups / std::max(groups, 1), 1, blocks);
+            const int per_split = (blocks + n_splits - 1) / n_splits;
+            n_splits = (blocks + per_split - 1) / per_split;
+            const size_t parts = static_cast<size_t>(n_single) * s.heads * n_splits;
+            float* ws_o = static_cast<float*>(ws.raw("latent_parts_o", parts * s.rank * sizeof(float)));
+            float* ws_ml = static_cast<float*>(ws.raw("latent_parts_ml", parts * 2 * sizeof(float)));
+            took(Path::AttentionLatentDecode);
+            kernel_check(celeg_latent_attention_fast(1, q_lat.data, static_cast<int>(q_lat.shape[1]), kv.k, kv.table, kv.table_stride,
+                                                     batch.cu_seqlens, batch.seq_slot, batch.seq_start, batch.n_seqs, 0,
+                                                     batch.token_slot, batch.positions, n_single, sink_p, out.data,
+                                                     static_cast<int>(out.shape[1]), ws_o, ws_ml, n_splits, per_split, s.heads,
+                                                     s.rank, s.rot, kv.page_tokens, kv.n_layers, kv.layer, scale, stream),
+                         "latent_attention (single tokens)");
+        }
+        if (T > n_single) {
+            const int max_tiles = (T - n_single) / 64 + std::max(batch.n_seqs - n_single, 1);
+            took(Path::AttentionLatentRows);
+            kernel_check(celeg_latent_attention_fast(0, q_lat.data, static_cast<int>(q_lat.shape[1]), kv.k, kv.table, kv.table_stride,
+                                                     batch.cu_seqlens, batch.seq_slot, batch.seq_start, batch.n_seqs, max_tiles,
+                                                     batch.token_slot, batch.positions, 0, sink_p, out.data,
+                                                     static_cast<int>(out.shape[1]), nullptr, nullptr, 1, 0, s.heads, s.rank,
+                                                     s.rot, kv.page_tokens, kv.n_layers, kv.layer, scale, stream),
+                         "latent_attention (rows)");
+        }
+        return;
+    }
     kernel_check(celeg_latent_attention(q_lat.data, static_cast<int>(q_lat.shape[1]), kv.k, dt(q_lat, "q_lat"), kv.table,
                                         kv.table_stride, batch.token_slot, batch.positions, sink ? sink->as<float>() : nullptr,
                                         out.data, static_cast<int>(out.shape[1]), batch.n_tokens, s.heads, s.rank, s.rot,

@@ -102,7 +102,7 @@ struct StepPrologue {
 // graph records; a replay counts nothing): what tests and tools ask to see that a size took the
 // path it was meant to take.
 enum class Path : int {
-    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, AttentionLatent, RoutedExperts, LinearF32, LinearLibrary, LinearStandIn,
+    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, AttentionLatent, AttentionLatentRows, AttentionLatentDecode, RoutedExperts, LinearF32, LinearLibrary, LinearStandIn,
     FusedSliced, FusedRows, FusedStaged, Tiled, TiledQkv, ArgmaxMerged, Count
 };
 const char* path_name(Path p);
@@ -123,6 +123,8 @@ public:
     int decode_split_rounds(long long groups, int rounds) const;
     bool decode_whole(long long groups, int rounds) const;
     bool attention_general = false;      // always the general attention kernel
+    bool use_latent_mfma = true;         // bfloat16 attention over a latent cache on the matrix cores
+    int latent_decode_workgroups = 512;  // single tokens: the keys are cut into shares until about this many workgroups run
     bool use_rope_table = true, use_argmax_parts = true, use_sliced = true, use_rows_kernel = true, use_tiles = true;
     bool use_qkv_tail = true;          // q/k/v products of many rows take norm, rotation and cache write along
     bool use_fresh_decode = true;      // decode-only steps: the attention prepares and writes the new keys and values
@@ -180,7 +182,7 @@ public:
                          const Tensor* gate);
     // q_lat [rows, heads * (rank + rot)] against the pages; out [rows, heads * rank]
     void latent_attention(const Tensor& q_lat, const Tensor& out, const LatentShape& shape, float scale, const Tensor* sink,
-                          const StepBatch& batch, const KVView& kv);
+                          const StepBatch& batch, const KVView& kv, Workspace& ws);
     // routed experts
     struct RoutePlan {
         Tensor ids, weights;                       // [rows * top]: expert and score of every (row, choice)

@@ -501,7 +501,7 @@ public:
         Tensor q_lat = rt.ws.buf("latent_q", rt.dtype, {T, H * D});
         rt.ops.headwise_linear(proj.cols(0, q_cols), static_cast<int>(qd), w_uk_t_->view, q_lat, static_cast<int>(D), shape_.rot, nullptr);
         Tensor o_lat = rt.ws.buf("latent_o", rt.dtype, {T, H * shape_.rank});
-        rt.ops.latent_attention(q_lat, o_lat, shape_, scale_, sink_ ? &sink_w_->view : nullptr, batch, *cache.kv);
+        rt.ops.latent_attention(q_lat, o_lat, shape_, scale_, sink_ ? &sink_w_->view : nullptr, batch, *cache.kv, rt.ws);
         Tensor heads = rt.ws.buf("latent_heads", rt.dtype, {T, H * vdim_});
         Tensor gate = gate_ ? proj.cols(q_cols + dkv_cols, g_cols) : Tensor();
         rt.ops.headwise_linear(o_lat, shape_.rank, uv_view_, heads, vdim_, 0, gate_ ? &gate : nullptr);

@@ -59,9 +59,16 @@ R3 = {"architecture": "Regipel", "vocab": 157, "width": 80, "streams": 1, "norm"
 R4 = {"architecture": "Regipel", "vocab": 260, "width": 128, "streams": 2, "norm": {"eps": 1e-5},
       "embedding": {"scale": 2.0}, "logit_scale": 0.5, "loop": {"start": 1, "stop": 2, "times": 3},
       "layers": [layer(mixer(2, 32, 32, 64, 64, base=100000.0), moe(8, 2, 64)) for _ in range(2)]}
-MODELS = {"R1": (R1, 11), "R2": (R2, 12), "R3": (R3, 13), "R4": (R4, 14)}
+# compressed rows that the matrix-core attention takes (a multiple of 16 values, rows of a multiple of
+# 8): 48 + 8 with five heads, and 128 + 24 with eighteen heads (two groups of heads for single tokens)
+R5 = {"architecture": "Regipel", "vocab": 190, "width": 64, "streams": 2, "norm": {"eps": 1e-5},
+      "embedding": {"scale": 1.3}, "logit_scale": 0.8,
+      "layers": [layer(mixer(5, 16, 8, 16, 48, base=700.0), moe(4, 2, 32)) for _ in range(2)]}
+R6 = {"architecture": "Regipel", "vocab": 175, "width": 64, "norm": {"eps": 1e-5}, "logit_scale": 1.5,
+      "layers": [layer(mixer(18, 8, 24, 8, 128, dims=16), None), layer(mixer(18, 8, 24, 8, 128, dims=16), moe(3, 1, 32))]}
+MODELS = {"R1": (R1, 11), "R2": (R2, 12), "R3": (R3, 13), "R4": (R4, 14), "R5": (R5, 15), "R6": (R6, 16)}
 LENGTHS = {"R1": [40, 57, 90, 128, 65, 33], "R2": [45, 130, 64, 100, 17, 33], "R3": [70, 33, 16, 97, 48, 15],
-           "R4": [31, 32, 150, 64, 49, 80]}
+           "R4": [31, 32, 150, 64, 49, 80], "R5": [63, 64, 65, 129, 20, 200], "R6": [70, 128, 13, 66, 191, 40]}
 SCHEDULES = {"whole": whole_schedule, "tail12": lambda reqs: tail_decode_schedule(reqs, tail=12),
              "portions": portions_schedule, "mixed": mixed_schedule}
 
@@ -157,7 +164,11 @@ def test_engine_matches_plain(folders, name, dtype, mode):
         assert_close(got[rid], ref[rid], dtype, f"{name}/{dtype}/{mode}/{rid}")
     lm.cache.check()
     assert lm.cache.n_free_slots == 4 and lm.cache.free_pages() == [max_tokens // 16] * len(lm.cache.free_pages())
-    assert lm.paths()["attention_latent"] > 0
+    paths = lm.paths()
+    assert paths["attention_latent"] > 0
+    fast = dtype == "bfloat16" and name in ("R4", "R5", "R6")
+    assert (paths["attention_latent_rows"] > 0) == fast
+    assert (paths["attention_latent_decode"] > 0) == (fast and mode != "whole")
     if any(l["mlp"] for l in MODELS[name][0]["layers"]):   # (every model here has some)
         assert lm.paths()["routed_experts"] > 0
 
@@ -235,16 +246,20 @@ def test_large_sinks(tmp_path, dtype):
         assert_close(got[rid], plain.model_logits(c, W, toks), dtype, f"sink/{rid}")
 
 
-def test_long_decoding_over_many_pages(folders):
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_over_many_pages(folders, dtype):
     """A short prompt, then 200 tokens one by one (steps replayed from a recorded graph), over a
-    dozen page borders."""
-    folder = folders("R4", "float32")
+    dozen page borders and, in bfloat16, over the borders of the blocks of 64 keys and of the
+    shares that the keys of a single token are cut into."""
+    folder = folders("R4", dtype)
     toks = random_tokens(R4["vocab"], 215, seed=77)
     steps = tail_decode_schedule({"long": toks}, tail=200)
-    lm, _ = load(folder, "float32", steps)
+    lm, _ = load(folder, dtype, steps)
+    if dtype == "bfloat16":
+        lm.set_knob("latent_decode_workgroups", 3)      # three shares of the keys
     got = EngineDriver(lm).run(steps)["long"]
     c, W = plain.load_model_folder(folder)
-    assert_close_f32(got, plain.model_logits(c, W, toks), "long decoding")
+    assert_close(got, plain.model_logits(c, W, toks), dtype, "long decoding")
     assert lm.runner.counters()["graph_replays"] > 100
 
 
