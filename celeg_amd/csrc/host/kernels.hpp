@@ -39,13 +39,15 @@ int celeg_latent_prepare(void* proj, int ld, int dtype, int q_off, int dkv_off, 
                          const int* positions, const int* token_slot, const int* table, int table_stride, void* pool,
                          int n_layers, int layer, int page_tokens, int write, int n_tokens, hipStream_t stream);
 int celeg_headwise_linear(const void* x, int ldx, int x_head, const void* w, int dtype, int heads, int N, int K, void* out,
-                          int ldo, int o_head, int tail, const void* gate, int ldg, int rows, hipStream_t stream);
+                          int ldo, int o_head, int tail, const void* gate, int ldg, int rows, int matrix_cores,
+                          hipStream_t stream);
 int celeg_latent_attention(const void* q, int ldq, const void* pool, int dtype, const int* table, int table_stride,
                            const int* token_slot, const int* positions, const float* sink, void* out, int ldo,
                            int n_tokens, int heads, int rank, int rot, int page_tokens, int n_layers, int layer,
                            float scale, hipStream_t stream);
 // latent_fast.hip
 int celeg_latent_attention_fast_ok(int rank, int rot);
+int celeg_latent_attention_tile_rows(int rank, int rot);
 int celeg_latent_attention_fast(int form, const void* q, int ldq, const void* pool, const int* table, int table_stride,
                                 const int* cu_seqlens, const int* seq_slot, const int* seq_start, int n_seqs, int max_tiles,
                                 const int* token_slot, const int* positions, int n_single, const float* sink, void* out,
@@ -54,13 +56,16 @@ int celeg_latent_attention_fast(int form, const void* q, int ldq, const void* po
 // moe.hip
 int celeg_moe_route(const float* logits, int rows, int experts, int top, int score, int renorm, int* ids, float* weights,
                     hipStream_t stream);
-int celeg_moe_tile_rows();
-int celeg_moe_plan(const int* ids, int n, int experts, int* offsets, int* place_of, int* entry_at, int* tile_expert,
+int celeg_moe_router(const void* x, int x_dtype, const float* w, int rows, int width, int experts, int top, int score,
+                     int renorm, int* ids, float* weights, hipStream_t stream);
+int celeg_moe_tile_rows(int matrix_cores);
+int celeg_moe_plan(const int* ids, int n, int experts, int tile_rows, int* offsets, int* place_of, int* entry_at, int* tile_expert,
                    int* tile_row0, int* n_tiles, hipStream_t stream);
 int celeg_moe_gather(const void* x, int dtype, const int* entry_at, const float* weights, void* a, int n, int top, int width,
                      hipStream_t stream);
 int celeg_moe_product(const void* a, const void* w, void* out, int dtype, int N, int K, int gated, const int* offsets,
-                      const int* tile_expert, const int* tile_row0, const int* n_tiles, int max_tiles, hipStream_t stream);
+                      const int* tile_expert, const int* tile_row0, const int* n_tiles, int max_tiles, int tile_rows,
+                      hipStream_t stream);
 int celeg_moe_combine(const void* y, int dtype, const int* place_of, const float* weights, void* out, int rows, int top,
                       int width, hipStream_t stream);
 // gemm_f32.hip

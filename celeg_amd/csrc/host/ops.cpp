@@ -198,9 +198,11 @@ void Ops::headwise_linear(const Tensor& x, int x_head, const Tensor& w, const Te
         ldg = rows_of(*gate, "gate");
         need(gate->shape[0] == x.shape[0] && gate->shape[1] == heads * N, "headwise_linear: gate must be [rows, heads * N]");
     }
+    const bool cores = moe_matrix_cores_ok(x.dtype, N, K) && ldx % 8 == 0 && x_head % 8 == 0 && ldo % 4 == 0 && o_head % 4 == 0 &&
+                       reinterpret_cast<uintptr_t>(x.data) % 16 == 0 && reinterpret_cast<uintptr_t>(out.data) % 8 == 0;
     kernel_check(celeg_headwise_linear(x.data, ldx, x_head, w.data, dt(x, "x"), static_cast<int>(heads), static_cast<int>(N),
                                        static_cast<int>(K), out.data, ldo, o_head, tail, gate ? gate->data : nullptr, ldg,
-                                       static_cast<int>(x.shape[0]), stream), "headwise_linear");
+                                       static_cast<int>(x.shape[0]), cores ? 1 : 0, stream), "headwise_linear");
 }
 
 void Ops::latent_attention(const Tensor& q_lat, const Tensor& out, const LatentShape& s, float scale, const Tensor* sink,
@@ -220,14 +222,15 @@ void Ops::latent_attention(const Tensor& q_lat, const Tensor& out, const LatentS
     latent_cache_fits(s, kv, q_lat.dtype, "latent_attention");
     took(Path::AttentionLatent);
     if (q_lat.dtype == DType::BF16 && use_latent_mfma && !attention_general && scale > 0.f && out.contiguous() &&
-        celeg_latent_attention_fast_ok(s.rank, s.rot)) {
+        celeg_latent_attention_fast_ok(s.rank, s.rot) && (kv.page_tokens & (kv.page_tokens - 1)) == 0) {
         const int T = batch.n_tokens, n_single = std::min(batch.single_rows, T);
         const float* sink_p = sink ? sink->as<float>() : nullptr;
         if (n_single > 0) {
             // single tokens: the keys of a row in shares, so that the chip is busy whatever the batch
             const int blocks = (std::max(hint_of(batch, kv), 1) + 63) / 64;
             const int groups = n_single * ((s.heads + 15) / 16);
-            int n_splits = std::clamp(latent_decode_workgroups / std::max(groups, 1), 1, blocks);
+            // (at most 64 shares, and a share is at least latent_decode_min_blocks blocks of 64 keys where there are that many)
+            int n_splits = std::clamp(latent_decode_workgroups / std::max(groups, 1), 1, std::min(64, std::max(1, blocks / std::max(latent_decode_min_blocks, 1))));
             const int per_split = (blocks + n_splits - 1) / n_splits;
             n_splits = (blocks + per_split - 1) / per_split;
             const size_t parts = static_cast<size_t>(n_single) * s.heads * n_splits;
@@ -242,7 +245,7 @@ void Ops::latent_attention(const Tensor& q_lat, const Tensor& out, const LatentS
                          "latent_attention (single tokens)");
         }
         if (T > n_single) {
-            const int max_tiles = (T - n_single) / 64 + std::max(batch.n_seqs - n_single, 1);
+            const int max_tiles = (T - n_single) / celeg_latent_attention_tile_rows(s.rank, s.rot) + std::max(batch.n_seqs - n_single, 1);
             took(Path::AttentionLatentRows);
             kernel_check(celeg_latent_attention_fast(0, q_lat.data, static_cast<int>(q_lat.shape[1]), kv.k, kv.table, kv.table_stride,
                                                      batch.cu_seqlens, batch.seq_slot, batch.seq_start, batch.n_seqs, max_tiles,
@@ -260,18 +263,14 @@ void Ops::latent_attention(const Tensor& q_lat, const Tensor& out, const LatentS
 }
 
 // ---------------------------------------------------------------------------- routed experts
-Ops::RoutePlan Ops::moe_route(const Tensor& logits, int top, int score, bool renorm, Workspace& ws) {
-    dev(logits, "logits", DType::F32);
-    need(logits.ndim == 2, "moe_route: logits must be [rows, experts]");
-    const long long rows = logits.shape[0], experts = logits.shape[1];
+static Ops::RoutePlan new_route_plan(long long rows, long long experts, int top, bool matrix_cores, Workspace& ws) {
     need(experts > 0 && experts <= 512, "moe_route: between 1 and 512 experts");
     need(top > 0 && top <= experts, "moe_route: `top` must be between 1 and the number of experts");
-    need(score == 0 || score == 1, "moe_route: score is sigmoid (0) or softmax (1)");
-    RoutePlan p;
+    Ops::RoutePlan p;
     p.n = static_cast<int>(rows * top);
     p.top = top;
     p.experts = static_cast<int>(experts);
-    const int tile = celeg_moe_tile_rows();
+    const int tile = p.tile_rows = celeg_moe_tile_rows(matrix_cores ? 1 : 0);
     p.max_tiles = static_cast<int>(std::min<long long>(p.n, p.n / tile + experts));
     const long long n = std::max(p.n, 1), tiles = std::max(p.max_tiles, 1);
     p.ids = ws.buf("moe_ids", DType::I32, {n});
@@ -282,11 +281,43 @@ Ops::RoutePlan Ops::moe_route(const Tensor& logits, int top, int score, bool ren
     p.tile_expert = ws.buf("moe_tile_expert", DType::I32, {tiles});
     p.tile_row0 = ws.buf("moe_tile_row0", DType::I32, {tiles});
     p.n_tiles = ws.buf("moe_n_tiles", DType::I32, {4});
-    took(Path::RoutedExperts);
-    kernel_check(celeg_moe_route(logits.as<float>(), static_cast<int>(rows), p.experts, top, score, renorm ? 1 : 0,
-                                 p.ids.as<int>(), p.weights.as<float>(), stream), "moe_route");
-    kernel_check(celeg_moe_plan(p.ids.as<int>(), p.n, p.experts, p.offsets.as<int>(), p.place_of.as<int>(), p.entry_at.as<int>(),
+    return p;
+}
+
+static void plan_of(const Ops::RoutePlan& p, hipStream_t stream) {
+    kernel_check(celeg_moe_plan(p.ids.as<int>(), p.n, p.experts, p.tile_rows, p.offsets.as<int>(), p.place_of.as<int>(), p.entry_at.as<int>(),
                                 p.tile_expert.as<int>(), p.tile_row0.as<int>(), p.n_tiles.as<int>(), stream), "moe_plan");
+}
+
+Ops::RoutePlan Ops::moe_route(const Tensor& logits, int top, int score, bool renorm, bool matrix_cores, Workspace& ws) {
+    dev(logits, "logits", DType::F32);
+    need(logits.ndim == 2, "moe_route: logits must be [rows, experts]");
+    need(score == 0 || score == 1, "moe_route: score is sigmoid (0) or softmax (1)");
+    RoutePlan p = new_route_plan(logits.shape[0], logits.shape[1], top, matrix_cores, ws);
+    took(Path::RoutedExperts);
+    kernel_check(celeg_moe_route(logits.as<float>(), static_cast<int>(logits.shape[0]), p.experts, top, score, renorm ? 1 : 0,
+                                 p.ids.as<int>(), p.weights.as<float>(), stream), "moe_route");
+    plan_of(p, stream);
+    return p;
+}
+
+Ops::RoutePlan Ops::moe_route_rows(const Tensor& x, const Tensor& router, int top, int score, bool renorm, bool matrix_cores,
+                                   Workspace& ws) {
+    dev(x, "x");
+    dev(router, "router", DType::F32);
+    need(x.ndim == 2 && x.contiguous() && router.ndim == 2 && router.shape[1] == x.shape[1], "moe_route_rows: x [rows, width], router [experts, width]");
+    need(score == 0 || score == 1, "moe_route_rows: score is sigmoid (0) or softmax (1)");
+    const long long rows = x.shape[0], width = x.shape[1], experts = router.shape[0];
+    if (!use_router_kernel || 4 * (width + experts) * 4 > 64 * 1024) {
+        Tensor logits = ws.buf("moe_logits", DType::F32, {rows, experts});
+        linear(x, router, logits, nullptr, ws);
+        return moe_route(logits, top, score, renorm, matrix_cores, ws);
+    }
+    RoutePlan p = new_route_plan(rows, experts, top, matrix_cores, ws);
+    took(Path::RoutedExperts);
+    kernel_check(celeg_moe_router(x.data, dt(x, "x"), router.as<float>(), static_cast<int>(rows), static_cast<int>(width), p.experts,
+                                  top, score, renorm ? 1 : 0, p.ids.as<int>(), p.weights.as<float>(), stream), "moe_router");
+    plan_of(p, stream);
     return p;
 }
 
@@ -306,9 +337,12 @@ void Ops::moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool 
     need(a.ndim == 2 && w.ndim == 2 && out.ndim == 2 && a.shape[0] == p.n && out.shape[0] == p.n && w.shape[1] == a.shape[1] &&
              w.shape[0] == static_cast<long long>(p.experts) * (gated ? 2 : 1) * out.shape[1],
          "moe_product: a [n, K], w [experts * N (* 2 if gated), K], out [n, N]");
+    need(a.contiguous() && w.contiguous() && out.contiguous(), "moe_product: a, w and out must be contiguous");
+    need(p.tile_rows == celeg_moe_tile_rows(0) || moe_matrix_cores_ok(a.dtype, out.shape[1], a.shape[1]),
+         "moe_product: the plan was made for the matrix cores, which do not take this product");
     kernel_check(celeg_moe_product(a.data, w.data, out.data, dt(a, "a"), static_cast<int>(out.shape[1]),
                                    static_cast<int>(a.shape[1]), gated ? 1 : 0, p.offsets.as<int>(), p.tile_expert.as<int>(),
-                                   p.tile_row0.as<int>(), p.n_tiles.as<int>(), p.max_tiles, stream), "moe_product");
+                                   p.tile_row0.as<int>(), p.n_tiles.as<int>(), p.max_tiles, p.tile_rows, stream), "moe_product");
 }
 
 void Ops::moe_combine(const Tensor& y, const RoutePlan& p, bool weighted, const Tensor& out) {

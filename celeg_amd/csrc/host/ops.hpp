@@ -123,8 +123,10 @@ public:
     int decode_split_rounds(long long groups, int rounds) const;
     bool decode_whole(long long groups, int rounds) const;
     bool attention_general = false;      // always the general attention kernel
+    bool use_router_kernel = true;       // the router's product inside the routing kernel
+    bool use_moe_mfma = true;            // bfloat16 products of routed experts and per-head matrices on the matrix cores
     bool use_latent_mfma = true;         // bfloat16 attention over a latent cache on the matrix cores
-    int latent_decode_workgroups = 512;  // single tokens: the keys are cut into shares until about this many workgroups run
+    int latent_decode_workgroups = 512, latent_decode_min_blocks = 1;  // single tokens: the keys are cut into shares until about this many workgroups run
     bool use_rope_table = true, use_argmax_parts = true, use_sliced = true, use_rows_kernel = true, use_tiles = true;
     bool use_qkv_tail = true;          // q/k/v products of many rows take norm, rotation and cache write along
     bool use_fresh_decode = true;      // decode-only steps: the attention prepares and writes the new keys and values
@@ -188,10 +190,19 @@ public:
         Tensor ids, weights;                       // [rows * top]: expert and score of every (row, choice)
         Tensor offsets, place_of, entry_at;        // rows sorted by expert
         Tensor tile_expert, tile_row0, n_tiles;
-        int n = 0, top = 0, experts = 0, max_tiles = 0;
+        int n = 0, top = 0, experts = 0, max_tiles = 0, tile_rows = 0;
     };
-    // logits [rows, experts] 32-bit -> the plan; score "sigmoid" (0) or "softmax" (1)
-    RoutePlan moe_route(const Tensor& logits, int top, int score, bool renorm, Workspace& ws);
+    // logits [rows, experts] 32-bit -> the plan; score "sigmoid" (0) or "softmax" (1); matrix_cores: the
+    // plan's products all run on the matrix cores (moe_matrix_cores_ok for each of them)
+    RoutePlan moe_route(const Tensor& logits, int top, int score, bool renorm, bool matrix_cores, Workspace& ws);
+    // the same from the rows themselves: x [rows, width] times the router's 32-bit matrix [experts, width],
+    // the product in 32-bit inside the routing kernel
+    RoutePlan moe_route_rows(const Tensor& x, const Tensor& router, int top, int score, bool renorm, bool matrix_cores,
+                             Workspace& ws);
+    // whether a product of experts [.., N, K] in this dtype runs on the matrix cores
+    bool moe_matrix_cores_ok(DType dtype, long long N, long long K) const {
+        return use_moe_mfma && dtype == DType::BF16 && K % 32 == 0 && N % 16 == 0;
+    }
     void moe_gather(const Tensor& x, const RoutePlan& plan, bool weighted, const Tensor& a);
     // out[p] = a[p] w[expert of p]^T; w [experts * N, K], or [experts * 2N, K] if gated (silu(gate) * up)
     void moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool gated, const RoutePlan& plan);

@@ -729,9 +729,9 @@ public:
     }
     Tensor forward(const Tensor& x, const StepBatch&, Runtime& rt) override {
         const long long T = x.shape[0];
-        Tensor logits = rt.ws.buf("moe_logits", DType::F32, {T, experts_});
-        rt.ops.linear(x, router_->view, logits, nullptr, rt.ws);
-        const Ops::RoutePlan plan = rt.ops.moe_route(logits, top_, score_, renorm_, rt.ws);
+        const bool cores = rt.ops.moe_matrix_cores_ok(x.dtype, ff_, width_) && rt.ops.moe_matrix_cores_ok(x.dtype, width_, ff_) &&
+                           w_gate_up_->view.dtype == x.dtype;
+        const Ops::RoutePlan plan = rt.ops.moe_route_rows(x, router_->view, top_, score_, renorm_, cores, rt.ws);
         Tensor a = rt.ws.buf("moe_in", rt.dtype, {T * top_, width_});
         rt.ops.moe_gather(x, plan, on_input_, a);
         Tensor act = rt.ws.buf("moe_act", rt.dtype, {T * top_, ff_});

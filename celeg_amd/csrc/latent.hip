@@ -5,6 +5,7 @@
 // dot product of q_lat with the cached row), the weighted sum runs over c, and W_uv is applied
 // to the result.  A learned number per head (the sink) may join the softmax's denominator; it
 // has no key and no value.
+#include "mfma_rows.h"
 #include "small_gemm.h"
 
 __device__ __forceinline__ size_t latent_row(int page, int n_layers, int layer, int page_tokens, int in_page, int row_dim) {
@@ -118,6 +119,47 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(const T* __restric
         }
 }
 
+// The same on the matrix cores (bfloat16; K a multiple of 32, N of 16, heads and rows 16-byte aligned).
+__global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(const __bf16* __restrict__ x, int ldx, int x_head,
+                                                                   const __bf16* __restrict__ w, int N, int K,
+                                                                   __bf16* __restrict__ out, int ldo, int o_head, int tail,
+                                                                   const __bf16* __restrict__ gate, int ldg, int rows) {
+    const int h = blockIdx.z, row0 = blockIdx.x * MR_ROWS;
+    const int rows_valid = min(MR_ROWS, rows - row0);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, qd = lane >> 4;
+    const int col0 = blockIdx.y * MR_COLS + wave * 16;
+    const __bf16* a = x + static_cast<size_t>(row0) * ldx + static_cast<size_t>(h) * x_head;
+    if (tail > 0 && blockIdx.y == 0)
+        for (int i = threadIdx.x; i < rows_valid * tail; i += 256) {
+            const int r = i / tail, j = i - r * tail;
+            out[static_cast<size_t>(row0 + r) * ldo + static_cast<size_t>(h) * o_head + N + j] = a[static_cast<size_t>(r) * ldx + K + j];
+        }
+    if (col0 >= N) return;
+    const __bf16* w0 = col0 + c < N ? w + (static_cast<size_t>(h) * N + col0 + c) * K : nullptr;
+    const __bf16* a_row[4];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) a_row[rt] = rt * 16 + c < rows_valid ? a + static_cast<size_t>(rt * 16 + c) * ldx : nullptr;
+    mr_f32x4 sums[1][4];
+    mfma_rows_product<1>(a_row, (rows_valid + 15) / 16, w0, nullptr, K, sums);
+    if (col0 + 4 * qd >= N) return;
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+        const int r = rt * 16 + c;
+        if (r >= rows_valid) continue;
+        mr_bf16x4 v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float s = sums[0][rt][j];
+            if (gate) {
+                const float g = static_cast<float>(gate[static_cast<size_t>(row0 + r) * ldg + static_cast<size_t>(h) * N + col0 + 4 * qd + j]);
+                s = static_cast<float>(static_cast<__bf16>(s)) * (1.0f / (1.0f + expf(-g)));
+            }
+            v[j] = static_cast<__bf16>(s);
+        }
+        *reinterpret_cast<mr_bf16x4*>(out + static_cast<size_t>(row0 + r) * ldo + static_cast<size_t>(h) * o_head + col0 + 4 * qd) = v;
+    }
+}
+
 // ---------------------------------------------------------------- attention, general form
 // One wavefront per (row, head).  The row's q_lat [rank + rot] against the cached rows of its
 // request at positions 0..pos, 64 keys at a time: a lane scores one key, the chunk joins a
@@ -216,8 +258,17 @@ extern "C" int celeg_latent_prepare(void* proj, int ld, int dtype, int q_off, in
 
 extern "C" int celeg_headwise_linear(const void* x, int ldx, int x_head, const void* w, int dtype, int heads, int N, int K,
                                      void* out, int ldo, int o_head, int tail, const void* gate, int ldg, int rows,
-                                     hipStream_t stream) {
+                                     int matrix_cores, hipStream_t stream) {
     if (rows <= 0) return 0;
+    if (matrix_cores) {
+        if (dtype != CELEG_BF16 || K % 32 || N % 16 || ldx % 8 || x_head % 8 || ldo % 4 || o_head % 4)
+            return static_cast<int>(hipErrorInvalidValue);
+        dim3 mgrid((rows + MR_ROWS - 1) / MR_ROWS, (N + MR_COLS - 1) / MR_COLS, heads);
+        hipLaunchKernelGGL(headwise_linear_mfma_kernel, mgrid, dim3(256), 0, stream, static_cast<const __bf16*>(x), ldx, x_head,
+                           static_cast<const __bf16*>(w), N, K, static_cast<__bf16*>(out), ldo, o_head, tail,
+                           static_cast<const __bf16*>(gate), ldg, rows);
+        return CELEG_LAUNCH_RESULT();
+    }
     dim3 grid((rows + SG_ROWS - 1) / SG_ROWS, (N + SG_COLS - 1) / SG_COLS, heads);
     if (dtype == CELEG_F32)
         hipLaunchKernelGGL(headwise_linear_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(x), ldx,

@@ -6,6 +6,7 @@
 //   product: out[p] = a[p] w[expert of p]^T over the tiles;
 //   combine: a row's `top` results summed (times the weight if it goes on the output).
 // Nothing is planned on the host: grids are sized by bounds, so a recorded step replays.
+#include "mfma_rows.h"
 #include "small_gemm.h"
 
 #define MOE_MAX_PER_LANE 8        // experts <= 512
@@ -13,10 +14,9 @@
 // ---------------------------------------------------------------- route
 // One wavefront per row.  score 0: sigmoid of the logit; 1: softmax over all experts.
 // The chosen experts' scores are the weights; with `renorm` they are divided by their sum.
-__global__ void moe_route_kernel(const float* __restrict__ logits, int experts, int top, int score, int renorm,
-                                 int* __restrict__ ids, float* __restrict__ weights) {
-    const int t = blockIdx.x, lane = threadIdx.x;
-    const float* z = logits + static_cast<size_t>(t) * experts;
+__device__ __forceinline__ void route_row(const float* z, int experts, int top, int score, int renorm, int* ids,
+                                          float* weights) {
+    const int lane = threadIdx.x & 63;
     float v[MOE_MAX_PER_LANE];
     float zmax = -INFINITY;
 #pragma unroll
@@ -56,12 +56,57 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int experts, 
         const float s = score == 1 ? expf(best - zmax) / denom : 1.0f / (1.0f + expf(-best));
         total += s;
         if (lane == 0) {
-            ids[static_cast<size_t>(t) * top + k] = best_e;
-            weights[static_cast<size_t>(t) * top + k] = s;
+            ids[k] = best_e;
+            weights[k] = s;
         }
     }
     if (renorm && lane == 0)
-        for (int k = 0; k < top; ++k) weights[static_cast<size_t>(t) * top + k] /= total;
+        for (int k = 0; k < top; ++k) weights[k] /= total;
+}
+
+__global__ void moe_route_kernel(const float* __restrict__ logits, int experts, int top, int score, int renorm,
+                                 int* __restrict__ ids, float* __restrict__ weights) {
+    const size_t t = blockIdx.x;
+    route_row(logits + t * experts, experts, top, score, renorm, ids + t * top, weights + t * top);
+}
+
+// The router's product and the choice in one kernel: a workgroup takes four rows, keeps them in LDS
+// in 32-bit, its wavefronts share out the experts (a weight is read once for the four rows; a row's
+// sum runs over k in an order that depends on nothing else), then each wavefront routes one row.
+#define ROUTE_ROWS 4
+template <typename TX>
+__global__ __launch_bounds__(256) void moe_router_kernel(const TX* __restrict__ x, const float* __restrict__ w, int rows,
+                                                         int width, int experts, int top, int score, int renorm,
+                                                         int* __restrict__ ids, float* __restrict__ weights) {
+    extern __shared__ float router_lds[];        // ROUTE_ROWS rows of width, then ROUTE_ROWS rows of logits
+    float* xs = router_lds;
+    float* zs = router_lds + ROUTE_ROWS * width;
+    const int row0 = blockIdx.x * ROUTE_ROWS;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < ROUTE_ROWS * width; i += 256) {
+        const int r = i / width;
+        xs[i] = row0 + r < rows ? to_float(x[static_cast<size_t>(row0) * width + i]) : 0.f;
+    }
+    __syncthreads();
+    for (int e = wave; e < experts; e += 4) {
+        const float* we = w + static_cast<size_t>(e) * width;
+        float acc[ROUTE_ROWS] = {0.f, 0.f, 0.f, 0.f};
+        for (int i = lane; i < width; i += CELEG_WAVE) {
+            const float wv = we[i];
+#pragma unroll
+            for (int r = 0; r < ROUTE_ROWS; ++r) acc[r] = fmaf(xs[r * width + i], wv, acc[r]);
+        }
+#pragma unroll
+        for (int r = 0; r < ROUTE_ROWS; ++r) {
+            const float total = wave_sum(acc[r]);
+            if (lane == 0) zs[r * experts + e] = total;
+        }
+    }
+    __syncthreads();
+    const int t = row0 + wave;
+    if (t < rows)
+        route_row(zs + wave * experts, experts, top, score, renorm, ids + static_cast<size_t>(t) * top,
+                  weights + static_cast<size_t>(t) * top);
 }
 
 // ---------------------------------------------------------------- plan
@@ -166,6 +211,48 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
     }
 }
 
+// The same on the matrix cores (bfloat16; tiles of 64 rows; K a multiple of 32, N of 16).
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_product_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w,
+                                                               __bf16* __restrict__ out, int N, int K,
+                                                               const int* __restrict__ offsets,
+                                                               const int* __restrict__ tile_expert,
+                                                               const int* __restrict__ tile_row0,
+                                                               const int* __restrict__ n_tiles) {
+    const int tile = blockIdx.x;
+    if (tile >= n_tiles[0]) return;
+    const int e = tile_expert[tile], row0 = tile_row0[tile];
+    const int rows_valid = min(MR_ROWS, offsets[e + 1] - row0);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, qd = lane >> 4;
+    const int col0 = blockIdx.y * MR_COLS + wave * 16;
+    if (col0 >= N) return;
+    const size_t per_expert = static_cast<size_t>(GATED ? 2 : 1) * N * K;
+    const __bf16* w0 = col0 + c < N ? w + static_cast<size_t>(e) * per_expert + static_cast<size_t>(col0 + c) * K : nullptr;
+    const __bf16* w1 = GATED && w0 ? w0 + static_cast<size_t>(N) * K : nullptr;
+    const __bf16* a_row[4];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) a_row[rt] = rt * 16 + c < rows_valid ? a + static_cast<size_t>(row0 + rt * 16 + c) * K : nullptr;
+    mr_f32x4 sums[GATED ? 2 : 1][4];
+    mfma_rows_product<GATED ? 2 : 1>(a_row, (rows_valid + 15) / 16, w0, w1, K, sums);
+    if (col0 + 4 * qd >= N) return;
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) {
+        if (rt * 16 + c >= rows_valid) continue;
+        mr_bf16x4 v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float x = sums[0][rt][r];
+            if (GATED) {
+                const float g = static_cast<float>(static_cast<__bf16>(x));
+                const float u = static_cast<float>(static_cast<__bf16>(sums[GATED ? 1 : 0][rt][r]));
+                x = (g / (1.0f + expf(-g))) * u;
+            }
+            v[r] = static_cast<__bf16>(x);
+        }
+        *reinterpret_cast<mr_bf16x4*>(out + static_cast<size_t>(row0 + rt * 16 + c) * N + col0 + 4 * qd) = v;
+    }
+}
+
 // ---------------------------------------------------------------- combine
 // out[t, :] = sum_k (weight of entry (t, k)) * y[place_of[t * top + k], :], summed in 32-bit
 template <typename T>
@@ -194,13 +281,31 @@ extern "C" int celeg_moe_route(const float* logits, int rows, int experts, int t
     return CELEG_LAUNCH_RESULT();
 }
 
-extern "C" int celeg_moe_tile_rows() { return SG_ROWS; }
+// rows of a tile: 64 where every product of the plan runs on the matrix cores, else 32
+// x [rows, width] (32-bit or bfloat16) times the router's 32-bit matrix w [experts, width], then the choice
+extern "C" int celeg_moe_router(const void* x, int x_dtype, const float* w, int rows, int width, int experts, int top,
+                                int score, int renorm, int* ids, float* weights, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    const size_t lds = static_cast<size_t>(ROUTE_ROWS) * (width + experts) * sizeof(float);
+    if (experts <= 0 || experts > MOE_MAX_PER_LANE * CELEG_WAVE || top <= 0 || top > experts || lds > 64 * 1024)
+        return static_cast<int>(hipErrorInvalidValue);
+    dim3 grid((rows + ROUTE_ROWS - 1) / ROUTE_ROWS);
+    if (x_dtype == CELEG_F32)
+        hipLaunchKernelGGL(moe_router_kernel<float>, grid, dim3(256), lds, stream, static_cast<const float*>(x), w, rows, width,
+                           experts, top, score, renorm, ids, weights);
+    else
+        hipLaunchKernelGGL(moe_router_kernel<bf16>, grid, dim3(256), lds, stream, static_cast<const bf16*>(x), w, rows, width,
+                           experts, top, score, renorm, ids, weights);
+    return CELEG_LAUNCH_RESULT();
+}
 
-extern "C" int celeg_moe_plan(const int* ids, int n, int experts, int* offsets, int* place_of, int* entry_at,
+extern "C" int celeg_moe_tile_rows(int matrix_cores) { return matrix_cores ? MR_ROWS : SG_ROWS; }
+
+extern "C" int celeg_moe_plan(const int* ids, int n, int experts, int tile_rows, int* offsets, int* place_of, int* entry_at,
                               int* tile_expert, int* tile_row0, int* n_tiles, hipStream_t stream) {
     if (n <= 0) return 0;
     const size_t lds = static_cast<size_t>(2 * experts + 1) * sizeof(int);
-    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), lds, stream, ids, n, experts, SG_ROWS, offsets, place_of,
+    hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), lds, stream, ids, n, experts, tile_rows, offsets, place_of,
                        entry_at, tile_expert, tile_row0, n_tiles);
     return CELEG_LAUNCH_RESULT();
 }
@@ -219,8 +324,22 @@ extern "C" int celeg_moe_gather(const void* x, int dtype, const int* entry_at, c
 
 extern "C" int celeg_moe_product(const void* a, const void* w, void* out, int dtype, int N, int K, int gated,
                                  const int* offsets, const int* tile_expert, const int* tile_row0, const int* n_tiles,
-                                 int max_tiles, hipStream_t stream) {
+                                 int max_tiles, int tile_rows, hipStream_t stream) {
     if (max_tiles <= 0) return 0;
+    if (tile_rows == MR_ROWS) {
+        if (dtype != CELEG_BF16 || K % 32 || N % 16) return static_cast<int>(hipErrorInvalidValue);
+        dim3 grid(max_tiles, (N + MR_COLS - 1) / MR_COLS);
+        if (gated)
+            hipLaunchKernelGGL(moe_product_mfma_kernel<true>, grid, dim3(256), 0, stream, static_cast<const __bf16*>(a),
+                               static_cast<const __bf16*>(w), static_cast<__bf16*>(out), N, K, offsets, tile_expert, tile_row0,
+                               n_tiles);
+        else
+            hipLaunchKernelGGL(moe_product_mfma_kernel<false>, grid, dim3(256), 0, stream, static_cast<const __bf16*>(a),
+                               static_cast<const __bf16*>(w), static_cast<__bf16*>(out), N, K, offsets, tile_expert, tile_row0,
+                               n_tiles);
+        return CELEG_LAUNCH_RESULT();
+    }
+    if (tile_rows != SG_ROWS) return static_cast<int>(hipErrorInvalidValue);
     dim3 grid(max_tiles, (N + SG_COLS - 1) / SG_COLS);
     if (dtype == CELEG_F32)
         hipLaunchKernelGGL(moe_product_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(a),

@@ -256,7 +256,8 @@ def test_long_decoding_over_many_pages(folders, dtype):
     steps = tail_decode_schedule({"long": toks}, tail=200)
     lm, _ = load(folder, dtype, steps)
     if dtype == "bfloat16":
-        lm.set_knob("latent_decode_workgroups", 3)      # three shares of the keys
+        lm.set_knob("latent_decode_workgroups", 3)      # three shares of the keys,
+        lm.set_knob("latent_decode_min_blocks", 1)      # however few the keys
     got = EngineDriver(lm).run(steps)["long"]
     c, W = plain.load_model_folder(folder)
     assert_close(got, plain.model_logits(c, W, toks), dtype, "long decoding")
