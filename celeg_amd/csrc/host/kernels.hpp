@@ -64,7 +64,7 @@ int celeg_moe_plan(const int* ids, int n, int experts, int tile_rows, int* offse
 int celeg_moe_gather(const void* x, int dtype, const int* entry_at, const float* weights, void* a, int n, int top, int width,
                      hipStream_t stream);
 int celeg_moe_product(const void* a, const void* w, void* out, int dtype, int N, int K, int gated, const int* offsets,
-                      const int* tile_expert, const int* tile_row0, const int* n_tiles, int max_tiles, int tile_rows,
+                      const int* tile_expert, const int* tile_row0, const int* n_tiles, int max_tiles, int tile_rows, int wide,
                       hipStream_t stream);
 int celeg_moe_combine(const void* y, int dtype, const int* place_of, const float* weights, void* out, int rows, int top,
                       int width, hipStream_t stream);

@@ -342,7 +342,8 @@ void Ops::moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool 
          "moe_product: the plan was made for the matrix cores, which do not take this product");
     kernel_check(celeg_moe_product(a.data, w.data, out.data, dt(a, "a"), static_cast<int>(out.shape[1]),
                                    static_cast<int>(a.shape[1]), gated ? 1 : 0, p.offsets.as<int>(), p.tile_expert.as<int>(),
-                                   p.tile_row0.as<int>(), p.n_tiles.as<int>(), p.max_tiles, p.tile_rows, stream), "moe_product");
+                                   p.tile_row0.as<int>(), p.n_tiles.as<int>(), p.max_tiles, p.tile_rows,
+                                   p.n >= 8 * p.experts ? 1 : 0, stream), "moe_product");
 }
 
 void Ops::moe_combine(const Tensor& y, const RoutePlan& p, bool weighted, const Tensor& out) {

@@ -135,12 +135,12 @@ __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(const __bf16*
             out[static_cast<size_t>(row0 + r) * ldo + static_cast<size_t>(h) * o_head + N + j] = a[static_cast<size_t>(r) * ldx + K + j];
         }
     if (col0 >= N) return;
-    const __bf16* w0 = col0 + c < N ? w + (static_cast<size_t>(h) * N + col0 + c) * K : nullptr;
+    const __bf16* w_row[1][1] = {{col0 + c < N ? w + (static_cast<size_t>(h) * N + col0 + c) * K : nullptr}};
     const __bf16* a_row[4];
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) a_row[rt] = rt * 16 + c < rows_valid ? a + static_cast<size_t>(rt * 16 + c) * ldx : nullptr;
-    mr_f32x4 sums[1][4];
-    mfma_rows_product<1>(a_row, (rows_valid + 15) / 16, w0, nullptr, K, sums);
+    mr_f32x4 sums[1][1][4];
+    mfma_rows_product<1, 1>(a_row, (rows_valid + 15) / 16, w_row, K, sums);
     if (col0 + 4 * qd >= N) return;
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) {
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(const __bf16*
         mr_bf16x4 v;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            float s = sums[0][rt][j];
+            float s = sums[0][0][rt][j];
             if (gate) {
                 const float g = static_cast<float>(gate[static_cast<size_t>(row0 + r) * ldg + static_cast<size_t>(h) * N + col0 + 4 * qd + j]);
                 s = static_cast<float>(static_cast<__bf16>(s)) * (1.0f / (1.0f + expf(-g)));

@@ -1,5 +1,5 @@
 // A tile product on the matrix cores for matrices picked per expert or per head (bfloat16):
-// a workgroup of four wavefronts computes 64 rows x 64 columns of a w^T, a wavefront 16 of the
+// a workgroup of four wavefronts computes 64 rows x 64 CT columns of a w^T, a wavefront 16 CT of the
 // columns for all the rows, operands straight from memory, sums in 32-bit, k in steps
 // of 32 in a fixed order.  The weights are the first operand, so that a lane ends up with four
 // neighbouring columns of one row.  K a multiple of 32; rows of a and w 16-byte aligned.
@@ -14,32 +14,37 @@ typedef unsigned int mr_u32x4 __attribute__((ext_vector_type(4)));
 #define MR_ROWS 64
 #define MR_COLS 64
 
-// sums[s][rt][r]: stream s (the weight rows w0 / w1), row rt * 16 + (lane & 15), column col0 + 4 (lane >> 4) + r,
-// col0 = 16 * wavefront.  a_row[rt]: this lane's row of a for row tile rt (null: none); w0 / w1: this
-// lane's weight row (column col0 + (lane & 15)) of each stream (null: none).
+// sums[s][ct][rt][r]: stream s, column tile ct of the wavefront, row rt * 16 + (lane & 15), column
+// (first column of the tile) + 4 (lane >> 4) + r.  a_row[rt]: this lane's row of a for row tile rt (null:
+// none); w_row[s][ct]: this lane's weight row (column of the tile + (lane & 15)) of stream s (null: none).
+// A wavefront with CT column tiles uses every operand of a it has loaded CT times.
 // K is walked in pieces of 128: a lane asks for 64 bytes in a run of each of its rows (its four
 // operands of the piece's four matrix instructions), all of a piece's loads before the first of its
 // products.  The values of k are thereby dealt to the instructions in another order than they lie in
 // (lane quad qd, instruction i of a piece: k0 + 32 qd + 8 i ..+8), the same order for both operands
 // and for every row, whatever else is in the batch.
-template <int STREAMS>
-__device__ __forceinline__ void mfma_rows_product(const __bf16* const (&a_row)[4], int row_tiles, const __bf16* w0,
-                                                  const __bf16* w1, int K, mr_f32x4 (&sums)[STREAMS][4]) {
+template <int STREAMS, int CT>
+__device__ __forceinline__ void mfma_rows_product(const __bf16* const (&a_row)[4], int row_tiles,
+                                                  const __bf16* const (&w_row)[STREAMS][CT], int K,
+                                                  mr_f32x4 (&sums)[STREAMS][CT][4]) {
     const int qd = (threadIdx.x & 63) >> 4;
 #pragma unroll
     for (int s = 0; s < STREAMS; ++s)
 #pragma unroll
-        for (int rt = 0; rt < 4; ++rt) sums[s][rt] = mr_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) sums[s][ct][rt] = mr_f32x4{0.f, 0.f, 0.f, 0.f};
     const mr_u32x4 zero = {0u, 0u, 0u, 0u};
     for (int k0 = 0; k0 < K; k0 += 128) {
         const int k = k0 + qd * 32;
-        mr_u32x4 wf[STREAMS][4], af[4][4];
+        mr_u32x4 wf[STREAMS][CT][4], af[4][4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const bool in = k + 8 * i < K;
-            wf[0][i] = in && w0 ? *reinterpret_cast<const mr_u32x4*>(w0 + k + 8 * i) : zero;
-            if (STREAMS > 1) wf[STREAMS - 1][i] = in && w1 ? *reinterpret_cast<const mr_u32x4*>(w1 + k + 8 * i) : zero;
-        }
+        for (int s = 0; s < STREAMS; ++s)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    wf[s][ct][i] = w_row[s][ct] && k + 8 * i < K ? *reinterpret_cast<const mr_u32x4*>(w_row[s][ct] + k + 8 * i) : zero;
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
@@ -50,9 +55,12 @@ __device__ __forceinline__ void mfma_rows_product(const __bf16* const (&a_row)[4
 #pragma unroll
             for (int s = 0; s < STREAMS; ++s)
 #pragma unroll
-                for (int rt = 0; rt < 4; ++rt)
-                    if (rt < row_tiles)
-                        sums[s][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mr_bf16x8, wf[s][i]),
-                                                                            __builtin_bit_cast(mr_bf16x8, af[rt][i]), sums[s][rt], 0, 0, 0);
+                for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                    for (int rt = 0; rt < 4; ++rt)
+                        if (rt < row_tiles)
+                            sums[s][ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mr_bf16x8, wf[s][ct][i]),
+                                                                                    __builtin_bit_cast(mr_bf16x8, af[rt][i]),
+                                                                                    sums[s][ct][rt], 0, 0, 0);
     }
 }

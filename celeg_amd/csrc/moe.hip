@@ -91,10 +91,24 @@ __global__ __launch_bounds__(256) void moe_router_kernel(const TX* __restrict__ 
     for (int e = wave; e < experts; e += 4) {
         const float* we = w + static_cast<size_t>(e) * width;
         float acc[ROUTE_ROWS] = {0.f, 0.f, 0.f, 0.f};
-        for (int i = lane; i < width; i += CELEG_WAVE) {
-            const float wv = we[i];
+        if ((width & 3) == 0) {
+            // four neighbouring weights a lane and load, several loads in flight
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll 4
+            for (int i = 4 * lane; i < width; i += 4 * CELEG_WAVE) {
+                const f32x4 wv = *reinterpret_cast<const f32x4*>(we + i);
 #pragma unroll
-            for (int r = 0; r < ROUTE_ROWS; ++r) acc[r] = fmaf(xs[r * width + i], wv, acc[r]);
+                for (int r = 0; r < ROUTE_ROWS; ++r) {
+                    const f32x4 xv = *reinterpret_cast<const f32x4*>(xs + r * width + i);
+                    acc[r] = fmaf(xv[3], wv[3], fmaf(xv[2], wv[2], fmaf(xv[1], wv[1], fmaf(xv[0], wv[0], acc[r]))));
+                }
+            }
+        } else {
+            for (int i = lane; i < width; i += CELEG_WAVE) {
+                const float wv = we[i];
+#pragma unroll
+                for (int r = 0; r < ROUTE_ROWS; ++r) acc[r] = fmaf(xs[r * width + i], wv, acc[r]);
+            }
         }
 #pragma unroll
         for (int r = 0; r < ROUTE_ROWS; ++r) {
@@ -211,45 +225,58 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
     }
 }
 
-// The same on the matrix cores (bfloat16; tiles of 64 rows; K a multiple of 32, N of 16).
-template <bool GATED>
-__global__ __launch_bounds__(256) void moe_product_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w,
-                                                               __bf16* __restrict__ out, int N, int K,
-                                                               const int* __restrict__ offsets,
-                                                               const int* __restrict__ tile_expert,
-                                                               const int* __restrict__ tile_row0,
-                                                               const int* __restrict__ n_tiles) {
+// The same on the matrix cores (bfloat16; K a multiple of 32, N of 16): tiles of 64 rows x 128 columns, a
+// wavefront two tiles of 16 columns, where the experts' tiles hold many rows (every operand of a used twice);
+// 64 columns, one tile a wavefront, where they hold few (a step of single tokens is bound by how many
+// workgroups pull the weights).
+template <bool GATED, int MOE_CT>
+__global__ __launch_bounds__(256, 2) void moe_product_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w,
+                                                                  __bf16* __restrict__ out, int N, int K,
+                                                                  const int* __restrict__ offsets,
+                                                                  const int* __restrict__ tile_expert,
+                                                                  const int* __restrict__ tile_row0,
+                                                                  const int* __restrict__ n_tiles) {
+    constexpr int S = GATED ? 2 : 1;
     const int tile = blockIdx.x;
     if (tile >= n_tiles[0]) return;
     const int e = tile_expert[tile], row0 = tile_row0[tile];
     const int rows_valid = min(MR_ROWS, offsets[e + 1] - row0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, qd = lane >> 4;
-    const int col0 = blockIdx.y * MR_COLS + wave * 16;
+    const int col0 = blockIdx.y * (MR_COLS * MOE_CT) + wave * 16 * MOE_CT;
     if (col0 >= N) return;
-    const size_t per_expert = static_cast<size_t>(GATED ? 2 : 1) * N * K;
-    const __bf16* w0 = col0 + c < N ? w + static_cast<size_t>(e) * per_expert + static_cast<size_t>(col0 + c) * K : nullptr;
-    const __bf16* w1 = GATED && w0 ? w0 + static_cast<size_t>(N) * K : nullptr;
+    const size_t per_expert = static_cast<size_t>(S) * N * K;
+    const __bf16* w_row[S][MOE_CT];
+#pragma unroll
+    for (int ct = 0; ct < MOE_CT; ++ct) {
+        const int col = col0 + ct * 16 + c;
+        w_row[0][ct] = col < N ? w + static_cast<size_t>(e) * per_expert + static_cast<size_t>(col) * K : nullptr;
+        if (GATED) w_row[S - 1][ct] = col < N ? w_row[0][ct] + static_cast<size_t>(N) * K : nullptr;
+    }
     const __bf16* a_row[4];
 #pragma unroll
     for (int rt = 0; rt < 4; ++rt) a_row[rt] = rt * 16 + c < rows_valid ? a + static_cast<size_t>(row0 + rt * 16 + c) * K : nullptr;
-    mr_f32x4 sums[GATED ? 2 : 1][4];
-    mfma_rows_product<GATED ? 2 : 1>(a_row, (rows_valid + 15) / 16, w0, w1, K, sums);
-    if (col0 + 4 * qd >= N) return;
+    mr_f32x4 sums[S][MOE_CT][4];
+    mfma_rows_product<S, MOE_CT>(a_row, (rows_valid + 15) / 16, w_row, K, sums);
 #pragma unroll
-    for (int rt = 0; rt < 4; ++rt) {
-        if (rt * 16 + c >= rows_valid) continue;
-        mr_bf16x4 v;
+    for (int ct = 0; ct < MOE_CT; ++ct) {
+        const int col = col0 + ct * 16 + 4 * qd;
+        if (col >= N) continue;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float x = sums[0][rt][r];
-            if (GATED) {
-                const float g = static_cast<float>(static_cast<__bf16>(x));
-                const float u = static_cast<float>(static_cast<__bf16>(sums[GATED ? 1 : 0][rt][r]));
-                x = (g / (1.0f + expf(-g))) * u;
+        for (int rt = 0; rt < 4; ++rt) {
+            if (rt * 16 + c >= rows_valid) continue;
+            mr_bf16x4 v;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float x = sums[0][ct][rt][r];
+                if (GATED) {
+                    const float g = static_cast<float>(static_cast<__bf16>(x));
+                    const float u = static_cast<float>(static_cast<__bf16>(sums[S - 1][ct][rt][r]));
+                    x = (g / (1.0f + expf(-g))) * u;
+                }
+                v[r] = static_cast<__bf16>(x);
             }
-            v[r] = static_cast<__bf16>(x);
+            *reinterpret_cast<mr_bf16x4*>(out + static_cast<size_t>(row0 + rt * 16 + c) * N + col) = v;
         }
-        *reinterpret_cast<mr_bf16x4*>(out + static_cast<size_t>(row0 + rt * 16 + c) * N + col0 + 4 * qd) = v;
     }
 }
 
@@ -324,19 +351,20 @@ extern "C" int celeg_moe_gather(const void* x, int dtype, const int* entry_at, c
 
 extern "C" int celeg_moe_product(const void* a, const void* w, void* out, int dtype, int N, int K, int gated,
                                  const int* offsets, const int* tile_expert, const int* tile_row0, const int* n_tiles,
-                                 int max_tiles, int tile_rows, hipStream_t stream) {
+                                 int max_tiles, int tile_rows, int wide, hipStream_t stream) {
     if (max_tiles <= 0) return 0;
     if (tile_rows == MR_ROWS) {
         if (dtype != CELEG_BF16 || K % 32 || N % 16) return static_cast<int>(hipErrorInvalidValue);
-        dim3 grid(max_tiles, (N + MR_COLS - 1) / MR_COLS);
-        if (gated)
-            hipLaunchKernelGGL(moe_product_mfma_kernel<true>, grid, dim3(256), 0, stream, static_cast<const __bf16*>(a),
-                               static_cast<const __bf16*>(w), static_cast<__bf16*>(out), N, K, offsets, tile_expert, tile_row0,
-                               n_tiles);
-        else
-            hipLaunchKernelGGL(moe_product_mfma_kernel<false>, grid, dim3(256), 0, stream, static_cast<const __bf16*>(a),
-                               static_cast<const __bf16*>(w), static_cast<__bf16*>(out), N, K, offsets, tile_expert, tile_row0,
-                               n_tiles);
+        const int ct = wide ? 2 : 1;
+        dim3 grid(max_tiles, (N + MR_COLS * ct - 1) / (MR_COLS * ct));
+#define MOE_GO(GATED, CT)                                                                                                       \
+    hipLaunchKernelGGL((moe_product_mfma_kernel<GATED, CT>), grid, dim3(256), 0, stream, static_cast<const __bf16*>(a),         \
+                       static_cast<const __bf16*>(w), static_cast<__bf16*>(out), N, K, offsets, tile_expert, tile_row0, n_tiles)
+        if (gated && wide) MOE_GO(true, 2);
+        else if (gated) MOE_GO(true, 1);
+        else if (wide) MOE_GO(false, 2);
+        else MOE_GO(false, 1);
+#undef MOE_GO
         return CELEG_LAUNCH_RESULT();
     }
     if (tile_rows != SG_ROWS) return static_cast<int>(hipErrorInvalidValue);
