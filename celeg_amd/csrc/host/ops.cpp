@@ -214,7 +214,7 @@ void Ops::latent_attention(const Tensor& q_lat, const Tensor& out, const LatentS
          "latent_attention: q_lat must be [rows, heads * (rank + rot)]");
     need(out.ndim == 2 && out.shape[0] == batch.n_tokens && out.shape[1] == static_cast<long long>(s.heads) * s.rank,
          "latent_attention: out must be [rows, heads * rank]");
-    need(s.rank <= 512, "latent_attention: a compressed row of more than 512 values does not fit the kernel's accumulators");
+    need(s.rank <= 1024, "latent_attention: a compressed row of more than 1,024 values does not fit the kernel's accumulators");
     if (sink) {
         dev(*sink, "sink", DType::F32);
         need(sink->numel() == s.heads, "latent_attention: one sink per head");

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(const __bf16*
 // request at positions 0..pos, 64 keys at a time: a lane scores one key, the chunk joins a
 // running (max, sum, accumulator) in 32-bit, the accumulator running over the first `rank`
 // values of the cached rows.  The chunking depends on the row's own position only.
-#define LAT_MAX_CHUNKS 8      // rank <= 512
+#define LAT_MAX_CHUNKS 16     // rank <= 1024
 
 template <typename T>
 __global__ void latent_attention_kernel(const T* __restrict__ q, int ldq, const T* __restrict__ pool,

@@ -225,8 +225,8 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
     }
 }
 
-// The same on the matrix cores (bfloat16; K a multiple of 32, N of 16): tiles of 64 rows x 128 columns, a
-// wavefront two tiles of 16 columns, where the experts' tiles hold many rows (every operand of a used twice);
+// The same on the matrix cores (bfloat16; K a multiple of 32, N of 16): tiles of 64 rows x 128 columns (256 for a
+// single stream of weights), a wavefront two (four) tiles of 16 columns, where the experts' tiles hold many rows (every operand of a used twice);
 // 64 columns, one tile a wavefront, where they hold few (a step of single tokens is bound by how many
 // workgroups pull the weights).
 template <bool GATED, int MOE_CT>
@@ -355,14 +355,14 @@ extern "C" int celeg_moe_product(const void* a, const void* w, void* out, int dt
     if (max_tiles <= 0) return 0;
     if (tile_rows == MR_ROWS) {
         if (dtype != CELEG_BF16 || K % 32 || N % 16) return static_cast<int>(hipErrorInvalidValue);
-        const int ct = wide ? 2 : 1;
+        const int ct = wide ? (gated ? 2 : 4) : 1;     // (one stream of weights leaves registers for four column tiles)
         dim3 grid(max_tiles, (N + MR_COLS * ct - 1) / (MR_COLS * ct));
 #define MOE_GO(GATED, CT)                                                                                                       \
     hipLaunchKernelGGL((moe_product_mfma_kernel<GATED, CT>), grid, dim3(256), 0, stream, static_cast<const __bf16*>(a),         \
                        static_cast<const __bf16*>(w), static_cast<__bf16*>(out), N, K, offsets, tile_expert, tile_row0, n_tiles)
         if (gated && wide) MOE_GO(true, 2);
         else if (gated) MOE_GO(true, 1);
-        else if (wide) MOE_GO(false, 2);
+        else if (wide) MOE_GO(false, 4);
         else MOE_GO(false, 1);
 #undef MOE_GO
         return CELEG_LAUNCH_RESULT();
