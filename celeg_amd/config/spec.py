@@ -43,6 +43,9 @@ class LayerSpec:
     # part with weights of its own ("hyper_connections": a "hyper_link" each)
     mixer_link: Optional[PartSpec] = None
     ffn_link: Optional[PartSpec] = None
+    # norms of the sub-layers' outputs, where the arrangement norms before and after ("sandwich_norm")
+    mixer_post_norm: Optional[PartSpec] = None
+    ffn_post_norm: Optional[PartSpec] = None
 
     def to_json(self) -> Dict[str, Any]:
         out = {"mixer": self.mixer.to_json(), "mixer_norm": self.mixer_norm.to_json(),
@@ -52,6 +55,10 @@ class LayerSpec:
             out["mixer_link"] = self.mixer_link.to_json()
         if self.ffn_link is not None:
             out["ffn_link"] = self.ffn_link.to_json()
+        if self.mixer_post_norm is not None:
+            out["mixer_post_norm"] = self.mixer_post_norm.to_json()
+        if self.ffn_post_norm is not None:
+            out["ffn_post_norm"] = self.ffn_post_norm.to_json()
         return out
 
     @classmethod
@@ -59,7 +66,8 @@ class LayerSpec:
         link = lambda key: PartSpec.from_json(l[key]) if l.get(key) else None
         return cls(PartSpec.from_json(l["mixer"]), PartSpec.from_json(l["mixer_norm"]),
                    PartSpec.from_json(l["ffn"]), PartSpec.from_json(l["ffn_norm"]),
-                   l.get("arrangement", "pre_norm"), link("mixer_link"), link("ffn_link"))
+                   l.get("arrangement", "pre_norm"), link("mixer_link"), link("ffn_link"),
+                   link("mixer_post_norm"), link("ffn_post_norm"))
 
 
 @dataclass(frozen=True)
@@ -67,9 +75,11 @@ class RunStep:
     """One entry of the run order.  ``layer`` indexes ``ModelSpec.layers`` (a layer may be named
     more than once: its weights are shared, its cache is not).  ``kv_from`` is the index of an
     EARLIER entry of the run order whose keys and values this entry's mixer reads instead of
-    writing its own."""
+    writing its own.  ``reinject``: before this entry the stream is replaced by the model's
+    ``reinjection`` part's mixture of the stream and the embedding's rows."""
     layer: int
     kv_from: Optional[int] = None
+    reinject: bool = False
 
 
 @dataclass(frozen=True)
@@ -86,23 +96,27 @@ class ModelSpec:
     eos_token_ids: Tuple[int, ...] = ()
     bos_token_id: Optional[int] = None
     streams: int = 1          # residual streams a row keeps between layers
+    reinjection: Optional[PartSpec] = None
 
     def to_json(self) -> Dict[str, Any]:
-        return {"architecture": self.architecture, "vocab_size": self.vocab_size,
+        out = {} if self.reinjection is None else {"reinjection": self.reinjection.to_json()}
+        return {**out, "architecture": self.architecture, "vocab_size": self.vocab_size,
                 "hidden_size": self.hidden_size, "max_context": self.max_context, "streams": self.streams,
                 "embedding": self.embedding.to_json(), "layers": [l.to_json() for l in self.layers],
-                "order": [{"layer": s.layer, "kv_from": s.kv_from} for s in self.order],
+                "order": [{"layer": s.layer, "kv_from": s.kv_from, **({"reinject": True} if s.reinject else {})}
+                          for s in self.order],
                 "final_norm": self.final_norm.to_json(), "head": self.head.to_json(),
                 "eos_token_ids": list(self.eos_token_ids), "bos_token_id": self.bos_token_id}
 
     @classmethod
     def from_json(cls, j: Dict[str, Any]) -> "ModelSpec":
         layers = tuple(LayerSpec.from_json(l) for l in j["layers"])
-        order = tuple(RunStep(s["layer"], s.get("kv_from")) for s in j["order"])
+        order = tuple(RunStep(s["layer"], s.get("kv_from"), bool(s.get("reinject"))) for s in j["order"])
         return cls(j["architecture"], j["vocab_size"], j["hidden_size"], j["max_context"],
                    PartSpec.from_json(j["embedding"]), layers, order, PartSpec.from_json(j["final_norm"]),
                    PartSpec.from_json(j["head"]), tuple(j.get("eos_token_ids") or ()), j.get("bos_token_id"),
-                   int(j.get("streams") or 1))
+                   int(j.get("streams") or 1),
+                   PartSpec.from_json(j["reinjection"]) if j.get("reinjection") else None)
 
     def tensor_names(self) -> List[str]:
         names: List[str] = []
@@ -111,9 +125,10 @@ class ModelSpec:
         return names
 
     def all_parts(self) -> List[PartSpec]:
-        parts = [self.embedding]
+        parts = [self.embedding] + ([self.reinjection] if self.reinjection is not None else [])
         for layer in self.layers:
             parts += [layer.mixer_norm, layer.mixer, layer.ffn_norm, layer.ffn]
-            parts += [p for p in (layer.mixer_link, layer.ffn_link) if p is not None]
+            parts += [p for p in (layer.mixer_link, layer.ffn_link, layer.mixer_post_norm, layer.ffn_post_norm)
+                      if p is not None]
         parts += [self.final_norm, self.head]
         return parts

@@ -35,7 +35,8 @@ HOST_FLAGS = ["-std=c++20", "-x", "hip", "-Wno-unused-result"] + COMMON_FLAGS
 LINK_FLAGS = ["-shared", "-fPIC", f"--offload-arch={ARCH}", "-ldl", "-lpthread"]
 # the kernel files, by the name tests and tools know them under
 MODULES = ["elementwise", "gemm_f32", "short_conv", "attention", "attention_fast", "gemv_fused", "gemv_slices",
-           "gemm_rows", "gemm_tiles", "sampling", "hyper", "latent", "latent_fast", "moe"]
+           "gemm_rows", "gemm_tiles", "sampling", "hyper", "latent", "latent_fast", "moe",
+           "norm_step", "sigmoid_attention", "delta_rule"]
 LIBRARY = "libceleg_amd"
 _lock = threading.Lock()
 

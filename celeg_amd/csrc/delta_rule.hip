@@ -1,0 +1,228 @@
+// The gated delta rule: a recurrent mixer whose state is a matrix per head.
+//
+// Per token and value head h (its query/key head g = h / (heads / kv_heads)), with unit key k,
+// scaled unit query q, value v, write strength beta and decay a (all 32-bit):
+//     S <- a S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q          S [dim, vdim]
+// The state S lives in the request's slot, in 32-bit, from token to token.
+//
+// Kernels:
+//  * delta_prepare: from the projections' rows, the short causal convolution of the q, k and v
+//    channels continuing from the request's saved inputs, silu, the unit norm of q and k per
+//    head, beta = sigmoid(.), a = exp(-exp(A_log) softplus(. + dt_bias));
+//  * delta_conv_state: the last taps - 1 inputs of every channel become the request's new state;
+//  * delta_scan: the recurrence, one wavefront per (request, value head, 64 columns of S): a lane
+//    owns a column of S, so the three sums over dim are the lane's own and no lane waits for another;
+//  * delta_gated_norm: o / rms(o) * w * silu(gate), per head.
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float dr_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float dr_silu(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float dr_softplus(float x) { return x > 20.0f ? x : log1pf(expf(x)); }
+
+// Input i' of channel c for the row whose place in its step's segment is `i` (row index t):
+// i' >= 0 lies in the step (row t - (i - i')), i' < 0 in the saved inputs (entry taps - 1 + i').
+template <typename T>
+__device__ __forceinline__ float conv_silu(const T* __restrict__ proj, int ld, int t, int i, int c, const float* __restrict__ w,
+                                           const float* __restrict__ saved, int n_channels, int taps) {
+    float y = 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j, ii = i - back;
+        const float x = ii >= 0 ? to_float(proj[static_cast<size_t>(t - back) * ld + c])
+                                : saved[static_cast<size_t>(taps - 1 + ii) * n_channels + c];
+        y = fmaf(w[static_cast<size_t>(c) * taps + j], x, y);
+    }
+    return dr_silu(y);
+}
+
+// One wavefront per (row, unit): units [0, G) are query heads, [G, 2G) key heads, [2G, 2G + H)
+// value heads, the last one computes beta and the decay of every value head.
+// proj columns: q [G*D] | k [G*D] | v [H*V] | (gate H*V, not read here) | b [H] at col_b | a [H] at col_a.
+// conv_w [2*G*D + H*V, taps]: the q, k and v channels' taps one after the other.
+template <typename T>
+__global__ __launch_bounds__(CELEG_WAVE) void delta_prepare_kernel(
+    const T* __restrict__ proj, int ld, int col_b, int col_a, const float* __restrict__ conv_w, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, const float* __restrict__ conv_state, size_t state_stride,
+    const int* __restrict__ positions, const int* __restrict__ token_seq, const int* __restrict__ seq_start,
+    const int* __restrict__ token_slot, float* __restrict__ qk, float* __restrict__ v_out, float* __restrict__ beta_decay, int G,
+    int H, int D, int V, int taps) {
+    const int t = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
+    const int n_channels = 2 * G * D + H * V;
+    if (unit == 2 * G + H) {
+        for (int h = lane; h < H; h += CELEG_WAVE) {
+            const float b = to_float(proj[static_cast<size_t>(t) * ld + col_b + h]);
+            const float a = to_float(proj[static_cast<size_t>(t) * ld + col_a + h]);
+            beta_decay[static_cast<size_t>(t) * 2 * H + h] = dr_sigmoid(b);
+            beta_decay[static_cast<size_t>(t) * 2 * H + H + h] = expf(-expf(a_log[h]) * dr_softplus(a + dt_bias[h]));
+        }
+        return;
+    }
+    const int i = positions[t] - seq_start[token_seq[t]];
+    const float* saved = conv_state + static_cast<size_t>(token_slot[t]) * state_stride;
+    if (unit >= 2 * G) {
+        const int h = unit - 2 * G;
+        for (int j = lane; j < V; j += CELEG_WAVE) {
+            const int c = 2 * G * D + h * V + j;
+            v_out[static_cast<size_t>(t) * H * V + h * V + j] = conv_silu(proj, ld, t, i, c, conv_w, saved, n_channels, taps);
+        }
+        return;
+    }
+    // a query or key head: unit vector over D (queries also times D^-1/2)
+    const int c0 = unit * D;
+    float* dst = qk + static_cast<size_t>(t) * 2 * G * D + c0;
+    float sum = 0.f;
+    for (int d = lane; d < D; d += CELEG_WAVE) {
+        const float x = conv_silu(proj, ld, t, i, c0 + d, conv_w, saved, n_channels, taps);
+        dst[d] = x;
+        sum += x * x;
+    }
+    sum = wave_sum(sum);
+    float inv = 1.0f / sqrtf(sum + 1e-6f);
+    if (unit < G) inv *= 1.0f / sqrtf(static_cast<float>(D));
+    for (int d = lane; d < D; d += CELEG_WAVE) dst[d] *= inv;     // (a lane reads what it wrote itself)
+}
+
+// per (request of the step, channel): new saved input j is old saved input j + n, or the step's
+// row j + n - (taps - 1) where that is not negative
+template <typename T>
+__global__ void delta_conv_state_kernel(const T* __restrict__ proj, int ld, float* __restrict__ conv_state, size_t state_stride,
+                                        const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot, int n_channels,
+                                        int taps) {
+    const int s = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= n_channels) return;
+    const int row0 = cu_seqlens[s], n = cu_seqlens[s + 1] - row0;
+    if (n <= 0) return;
+    float* saved = conv_state + static_cast<size_t>(seq_slot[s]) * state_stride;
+    for (int j = 0; j < taps - 1; ++j) {      // rising j: entry j + n is still the old one when j is written
+        const int from = j + n - (taps - 1);
+        saved[static_cast<size_t>(j) * n_channels + c] =
+            from >= 0 ? to_float(proj[static_cast<size_t>(row0 + from) * ld + c]) : saved[static_cast<size_t>(j + n) * n_channels + c];
+    }
+}
+
+// One wavefront per (request, value head, 64 columns).  S's columns of this wavefront sit in LDS
+// as [D][64]; k and q of the token are staged in LDS for all lanes to read.
+__global__ __launch_bounds__(CELEG_WAVE) void delta_scan_kernel(
+    const float* __restrict__ qk, const float* __restrict__ v, const float* __restrict__ beta_decay, float* __restrict__ state,
+    size_t state_stride, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot, float* __restrict__ out, int G, int H,
+    int D, int V) {
+    extern __shared__ float lds[];       // S [D][64], k [D], q [D]
+    float* S = lds;
+    float* ks = lds + static_cast<size_t>(D) * CELEG_WAVE;
+    float* qs = ks + D;
+    const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int j = blockIdx.z * CELEG_WAVE + lane;
+    const bool live = j < V;
+    const int g = h / (H / G);
+    const int row0 = cu_seqlens[s], n = cu_seqlens[s + 1] - row0;
+    if (n <= 0) return;
+    float* mine = state + static_cast<size_t>(seq_slot[s]) * state_stride + static_cast<size_t>(h) * D * V;
+    for (int d = 0; d < D; ++d) S[d * CELEG_WAVE + lane] = live ? mine[static_cast<size_t>(d) * V + j] : 0.f;
+    for (int r = 0; r < n; ++r) {
+        const size_t t = static_cast<size_t>(row0 + r);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (int d = lane; d < D; d += CELEG_WAVE) {
+            qs[d] = qk[t * 2 * G * D + static_cast<size_t>(g) * D + d];
+            ks[d] = qk[t * 2 * G * D + static_cast<size_t>(G + g) * D + d];
+        }
+        const float beta = beta_decay[t * 2 * H + h], decay = beta_decay[t * 2 * H + H + h];
+        const float vj = live ? v[t * H * V + static_cast<size_t>(h) * V + j] : 0.f;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        float kv = 0.f;
+        for (int d = 0; d < D; ++d) {
+            const float sd = decay * S[d * CELEG_WAVE + lane];
+            S[d * CELEG_WAVE + lane] = sd;
+            kv = fmaf(ks[d], sd, kv);
+        }
+        const float u = beta * (vj - kv);
+        float o = 0.f;
+        for (int d = 0; d < D; ++d) {
+            const float sd = fmaf(ks[d], u, S[d * CELEG_WAVE + lane]);
+            S[d * CELEG_WAVE + lane] = sd;
+            o = fmaf(qs[d], sd, o);
+        }
+        if (live) out[t * H * V + static_cast<size_t>(h) * V + j] = o;
+    }
+    if (live)
+        for (int d = 0; d < D; ++d) mine[static_cast<size_t>(d) * V + j] = S[d * CELEG_WAVE + lane];
+}
+
+// one wavefront per (row, head): out = o / sqrt(mean(o^2) + eps) * w * silu(gate)
+template <typename T>
+__global__ __launch_bounds__(CELEG_WAVE) void delta_gated_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                                                      const T* __restrict__ gate, int ldg, float eps,
+                                                                      T* __restrict__ out, int H, int V) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float* row = o + (static_cast<size_t>(t) * H + h) * V;
+    float sum = 0.f;
+    for (int j = lane; j < V; j += CELEG_WAVE) sum += row[j] * row[j];
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sqrtf(sum / static_cast<float>(V) + eps);
+    for (int j = lane; j < V; j += CELEG_WAVE) {
+        const float z = to_float(gate[static_cast<size_t>(t) * ldg + h * V + j]);
+        out[(static_cast<size_t>(t) * H + h) * V + j] = from_float<T>(row[j] * inv * w[j] * dr_silu(z));
+    }
+}
+
+}  // namespace
+
+extern "C" int celeg_delta_prepare(const void* proj, int ld, int dtype, int col_b, int col_a, const float* conv_w,
+                                   const float* a_log, const float* dt_bias, const float* conv_state, size_t state_stride,
+                                   const int* positions, const int* token_seq, const int* seq_start, const int* token_slot,
+                                   float* qk, float* v_out, float* beta_decay, int n_tokens, int G, int H, int D, int V, int taps,
+                                   hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    dim3 grid(n_tokens, 2 * G + H + 1), block(CELEG_WAVE);
+    if (dtype == CELEG_F32)
+        hipLaunchKernelGGL(delta_prepare_kernel<float>, grid, block, 0, stream, static_cast<const float*>(proj), ld, col_b, col_a,
+                           conv_w, a_log, dt_bias, conv_state, state_stride, positions, token_seq, seq_start, token_slot, qk,
+                           v_out, beta_decay, G, H, D, V, taps);
+    else
+        hipLaunchKernelGGL(delta_prepare_kernel<bf16>, grid, block, 0, stream, static_cast<const bf16*>(proj), ld, col_b, col_a,
+                           conv_w, a_log, dt_bias, conv_state, state_stride, positions, token_seq, seq_start, token_slot, qk,
+                           v_out, beta_decay, G, H, D, V, taps);
+    return CELEG_LAUNCH_RESULT();
+}
+
+extern "C" int celeg_delta_conv_state(const void* proj, int ld, int dtype, float* conv_state, size_t state_stride,
+                                      const int* cu_seqlens, const int* seq_slot, int n_seqs, int n_channels, int taps,
+                                      hipStream_t stream) {
+    if (n_seqs <= 0 || taps <= 1) return 0;
+    dim3 grid((n_channels + 255) / 256, n_seqs), block(256);
+    if (dtype == CELEG_F32)
+        hipLaunchKernelGGL(delta_conv_state_kernel<float>, grid, block, 0, stream, static_cast<const float*>(proj), ld, conv_state,
+                           state_stride, cu_seqlens, seq_slot, n_channels, taps);
+    else
+        hipLaunchKernelGGL(delta_conv_state_kernel<bf16>, grid, block, 0, stream, static_cast<const bf16*>(proj), ld, conv_state,
+                           state_stride, cu_seqlens, seq_slot, n_channels, taps);
+    return CELEG_LAUNCH_RESULT();
+}
+
+extern "C" int celeg_delta_scan(const float* qk, const float* v, const float* beta_decay, float* state, size_t state_stride,
+                                const int* cu_seqlens, const int* seq_slot, float* out, int n_seqs, int G, int H, int D, int V,
+                                hipStream_t stream) {
+    if (n_seqs <= 0) return 0;
+    const size_t lds = (static_cast<size_t>(D) * CELEG_WAVE + 2 * static_cast<size_t>(D)) * sizeof(float);
+    if (lds > 64 * 1024 || H % G) return static_cast<int>(hipErrorInvalidValue);
+    dim3 grid(n_seqs, H, (V + CELEG_WAVE - 1) / CELEG_WAVE), block(CELEG_WAVE);
+    hipLaunchKernelGGL(delta_scan_kernel, grid, block, lds, stream, qk, v, beta_decay, state, state_stride, cu_seqlens, seq_slot,
+                       out, G, H, D, V);
+    return CELEG_LAUNCH_RESULT();
+}
+
+extern "C" int celeg_delta_gated_norm(const float* o, const float* w, const void* gate, int ldg, int dtype, float eps, void* out,
+                                      int n_tokens, int H, int V, hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    dim3 grid(n_tokens, H), block(CELEG_WAVE);
+    if (dtype == CELEG_F32)
+        hipLaunchKernelGGL(delta_gated_norm_kernel<float>, grid, block, 0, stream, o, w, static_cast<const float*>(gate), ldg, eps,
+                           static_cast<float*>(out), H, V);
+    else
+        hipLaunchKernelGGL(delta_gated_norm_kernel<bf16>, grid, block, 0, stream, o, w, static_cast<const bf16*>(gate), ldg, eps,
+                           static_cast<bf16*>(out), H, V);
+    return CELEG_LAUNCH_RESULT();
+}

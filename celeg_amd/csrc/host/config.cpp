@@ -613,6 +613,211 @@ ModelSpec regipel_build_spec(const Json& c) {
 
 }  // namespace
 
+// ---------------------------------------------------------------------------- Kifetar
+// A decoder that norms every sub-layer's input and output (layer norms with weight and bias),
+// mixes by attention with sigmoid weights inside a sliding window or by a gated delta rule, and
+// may run a range of its layers several times, taking the embedding's rows in again before
+// every run of the range.  config.json describes every layer by itself:
+//   {"architecture": "Kifetar", "vocab", "width", "norm": {"eps"},
+//    "loop": {"start", "stop", "times"} (layers start..stop-1 run `times` times in a row with the
+//    same weights and a cache or state of their own each time; before the first layer of every
+//    such run the stream becomes W_in [stream ; embedding rows], tensor "loop.in"),
+//    "max_context" (an engine limit; optional),
+//    "layers": [{"type": "attention",
+//                "mixer": {"heads", "kv_heads", "dim", "vdim" (= dim: the values are the keys as
+//                          projected), "scale", "mask": {"size"} (absent: every earlier key),
+//                          "rot": {"base", "dims", "scaling": {"factor", "low", "high", "original"}}
+//                          (absent, or dims 0: no rotation; scaling optional)},
+//                "mlp": null | {"kind": "dense", "ff"}},
+//               {"type": "delta", "mixer": {"heads", "kv_heads", "dim", "vdim", "conv"}, "mlp": ...}]}
+// The output head is the embedding table.
+// Tensors: embed, loop.in, final.norm(.b), l<i>.norm1|norm1b|norm2|norm2b(.b),
+// attention: l<i>.mix.{q, q.b, k, k.b, q.norm, k.norm, temp, pb, g, o};
+// delta: l<i>.mix.{q, q.conv, k, k.conv, v, v.conv, b, a, A_log, dt_bias, norm, g, o};
+// l<i>.mlp.{gate, up, down}.
+namespace {
+
+Json kifetar_read_config(const Json& raw, const TensorShapes*) {
+    if (!raw.is_object()) throw ConfigError("config.json is not an object");
+    Json out = Json::object();
+    out.set("architecture", "Kifetar");
+    out.set("vocab", regipel_int(raw, "vocab", ""));
+    const long long width = regipel_int(raw, "width", "");
+    out.set("width", width);
+    const double eps = regipel_number(regipel_object(raw, "norm", ""), "eps", "norm.");
+    if (!(eps > 0)) throw ConfigError("config.json: 'norm.eps' must be positive");
+    out.set("norm", Json::object().set("eps", eps));
+    out.set("max_context", raw["max_context"].is_null() ? 131072LL : regipel_int(raw, "max_context", ""));
+    if (!raw["layers"].is_array() || raw["layers"].size() == 0) throw ConfigError("config.json: 'layers' must be a list of layers");
+    Json layers = Json::array();
+    int i = 0;
+    for (const Json& l : raw["layers"].items()) {
+        const std::string where = "layers[" + std::to_string(i++) + "].";
+        if (!l.is_object()) throw ConfigError("config.json: " + where + " must be an object");
+        const std::string type = l.get_string("type", "");
+        const Json& m = regipel_object(l, "mixer", where);
+        const std::string mw = where + "mixer.";
+        Json mixer = Json::object();
+        const long long heads = regipel_int(m, "heads", mw), kv_heads = regipel_int(m, "kv_heads", mw);
+        if (heads % kv_heads) throw ConfigError("config.json: " + mw + "'heads' must be a multiple of 'kv_heads'");
+        mixer.set("heads", heads).set("kv_heads", kv_heads).set("dim", regipel_int(m, "dim", mw)).set("vdim", regipel_int(m, "vdim", mw));
+        if (type == "attention") {
+            if (mixer["vdim"].as_int() != mixer["dim"].as_int())
+                throw ConfigError("config.json: " + mw + "'vdim' must equal 'dim': the values are the keys as projected");
+            if (mixer["dim"].as_int() % 2) throw ConfigError("config.json: " + mw + "'dim' must be even");
+            mixer.set("scale", regipel_number(m, "scale", mw));
+            mixer.set("mask", m["mask"].is_null() ? Json() : Json::object().set("size", regipel_int(regipel_object(m, "mask", mw), "size", mw + "mask.")));
+            Json rot;
+            if (!m["rot"].is_null()) {
+                const Json& r = regipel_object(m, "rot", mw);
+                const long long dims = regipel_int(r, "dims", mw + "rot.", 0);
+                if (dims % 2 || dims > mixer["dim"].as_int()) throw ConfigError("config.json: " + mw + "'rot.dims' must be even and at most 'dim'");
+                if (dims > 0) {
+                    const double base = regipel_number(r, "base", mw + "rot.");
+                    if (!(base > 0)) throw ConfigError("config.json: " + mw + "'rot.base' must be positive");
+                    rot = Json::object().set("base", base).set("dims", dims);
+                    if (!r["scaling"].is_null()) {
+                        const Json& sc = regipel_object(r, "scaling", mw + "rot.");
+                        const std::string sw = mw + "rot.scaling.";
+                        Json scaling = Json::object();
+                        for (const char* key : {"factor", "low", "high", "original"}) scaling.set(key, regipel_number(sc, key, sw));
+                        if (!(scaling["factor"].as_double() > 0) || !(scaling["low"].as_double() > 0) ||
+                            !(scaling["high"].as_double() > scaling["low"].as_double()) || !(scaling["original"].as_double() > 0))
+                            throw ConfigError("config.json: " + sw + " needs factor > 0, 0 < low < high and original > 0");
+                        rot.set("scaling", scaling);
+                    }
+                }
+            }
+            mixer.set("rot", rot);
+        } else if (type == "delta") {
+            mixer.set("conv", regipel_int(m, "conv", mw));
+        } else {
+            throw ConfigError("config.json: " + where + "'type' is '" + type + "'; known types are ['attention', 'delta']");
+        }
+        Json mlp;
+        if (!l["mlp"].is_null()) {
+            const Json& f = regipel_object(l, "mlp", where);
+            const std::string kind = f.get_string("kind", "");
+            if (kind != "dense") throw ConfigError("config.json: " + where + "mlp.'kind' is '" + kind + "'; known kinds are ['dense']");
+            mlp = Json::object().set("kind", kind).set("ff", regipel_int(f, "ff", where + "mlp."));
+        }
+        layers.push(Json::object().set("type", type).set("mixer", mixer).set("mlp", mlp));
+    }
+    out.set("layers", layers);
+    const long long n_layers = static_cast<long long>(layers.size());
+    long long start = 0, stop = 0, times = 1;
+    if (!raw["loop"].is_null()) {
+        const Json& loop = regipel_object(raw, "loop", "");
+        start = regipel_int(loop, "start", "loop.", 0);
+        stop = regipel_int(loop, "stop", "loop.", 0);
+        times = regipel_int(loop, "times", "loop.", 0);
+        if (start > stop || stop > n_layers)
+            throw ConfigError("config.json: 'loop' must satisfy 0 <= start <= stop <= " + std::to_string(n_layers));
+    }
+    out.set("loop", Json::object().set("start", start).set("stop", stop).set("times", times));
+    for (const char* key : {"bos_token_id", "eos_token_id"})
+        if (!raw[key].is_null()) out.set(key, raw[key]);
+    return out;
+}
+
+ModelSpec kifetar_build_spec(const Json& c) {
+    const long long W = c["width"].as_int();
+    const double eps = c["norm"]["eps"].as_double();
+    auto norm = [&](const std::string& name) {
+        PartSpec p;
+        p.kind = "layernorm";
+        p.params = Json::object().set("width", W).set("eps", eps).set("bias", true);
+        p.tensors = {{"weight", name}, {"bias", name + ".b"}};
+        return p;
+    };
+    ModelSpec spec;
+    int i = 0;
+    for (const Json& l : c["layers"].items()) {
+        const std::string p = "l" + std::to_string(i) + ".";
+        const Json& m = l["mixer"];
+        LayerSpec layer;
+        layer.arrangement = "sandwich_norm";
+        if (l["type"].as_string() == "attention") {
+            layer.mixer.kind = "sigmoid_attention";
+            layer.mixer.params = Json::object().set("width", W).set("heads", m["heads"]).set("kv_heads", m["kv_heads"])
+                                     .set("head_dim", m["dim"]).set("scale", m["scale"]).set("eps", eps).set("qk_norm", true)
+                                     .set("bias", true).set("values", "keys").set("temperature", true).set("score_bias", true)
+                                     .set("head_gate", true);
+            if (!m["mask"].is_null()) layer.mixer.params.set("window", m["mask"]["size"]);
+            if (!m["rot"].is_null()) {
+                PartSpec rope;
+                rope.kind = "rope";
+                rope.params = Json::object().set("theta", m["rot"]["base"]).set("rotary_dim", m["rot"]["dims"])
+                                  .set("head_dim", m["dim"]).set("pairing", "halves");
+                if (!m["rot"]["scaling"].is_null()) rope.params.set("scaling", m["rot"]["scaling"]);
+                layer.mixer.params.set("position", rope.to_json());
+            }
+            layer.mixer.tensors = {{"q", p + "mix.q"},           {"k", p + "mix.k"},           {"o", p + "mix.o"},
+                                   {"q_bias", p + "mix.q.b"},    {"k_bias", p + "mix.k.b"},    {"q_norm", p + "mix.q.norm"},
+                                   {"k_norm", p + "mix.k.norm"}, {"temp", p + "mix.temp"},     {"pb", p + "mix.pb"},
+                                   {"g", p + "mix.g"}};
+        } else {
+            layer.mixer.kind = "gated_delta_rule";
+            layer.mixer.params = Json::object().set("width", W).set("heads", m["heads"]).set("kv_heads", m["kv_heads"])
+                                     .set("dim", m["dim"]).set("vdim", m["vdim"]).set("taps", m["conv"]).set("eps", eps);
+            layer.mixer.tensors = {{"q", p + "mix.q"},   {"k", p + "mix.k"},         {"v", p + "mix.v"},
+                                   {"q_conv", p + "mix.q.conv"}, {"k_conv", p + "mix.k.conv"}, {"v_conv", p + "mix.v.conv"},
+                                   {"b", p + "mix.b"},   {"a", p + "mix.a"},         {"A_log", p + "mix.A_log"},
+                                   {"dt_bias", p + "mix.dt_bias"}, {"norm", p + "mix.norm"}, {"g", p + "mix.g"},
+                                   {"o", p + "mix.o"}};
+        }
+        layer.mixer_norm = norm(p + "norm1");
+        layer.mixer_post_norm = norm(p + "norm1b");
+        if (l["mlp"].is_null()) {
+            layer.ffn.kind = "none";
+            layer.ffn_norm.kind = "identity";
+        } else {
+            layer.ffn.kind = "swiglu";
+            layer.ffn.params = Json::object().set("width", W).set("ff", l["mlp"]["ff"]);
+            layer.ffn.tensors = {{"gate", p + "mlp.gate"}, {"up", p + "mlp.up"}, {"down", p + "mlp.down"}};
+            layer.ffn_norm = norm(p + "norm2");
+            layer.ffn_post_norm = norm(p + "norm2b");
+        }
+        spec.layers.push_back(std::move(layer));
+        ++i;
+    }
+    const int n_layers = i;
+    const int start = static_cast<int>(c["loop"]["start"].as_int()), stop = static_cast<int>(c["loop"]["stop"].as_int());
+    const int times = static_cast<int>(c["loop"]["times"].as_int());
+    for (int l = 0; l < start; ++l) spec.order.push_back(RunStep{l, {}, false});
+    bool reinjects = false;
+    for (int pass = 0; pass < times; ++pass)
+        for (int l = start; l < stop; ++l) {
+            spec.order.push_back(RunStep{l, {}, l == start});
+            reinjects = true;
+        }
+    for (int l = stop; l < n_layers; ++l) spec.order.push_back(RunStep{l, {}, false});
+    if (reinjects) {
+        spec.reinjection.kind = "linear_concat";
+        spec.reinjection.params = Json::object().set("width", W);
+        spec.reinjection.tensors = {{"weight", "loop.in"}};
+    }
+    spec.architecture = "Kifetar";
+    spec.vocab_size = static_cast<int>(c["vocab"].as_int());
+    spec.hidden_size = static_cast<int>(W);
+    spec.max_context = static_cast<int>(c["max_context"].as_int());
+    spec.embedding.kind = "embedding";
+    spec.embedding.params = Json::object().set("vocab", c["vocab"]).set("width", W);
+    spec.embedding.tensors = {{"table", "embed"}};
+    spec.head.kind = "tied_head";
+    spec.head.params = Json::object().set("vocab", c["vocab"]).set("width", W);
+    spec.final_norm = norm("final.norm");
+    if (c["eos_token_id"].is_array())
+        for (const Json& e : c["eos_token_id"].items()) spec.eos_token_ids.push_back(static_cast<int>(e.as_int()));
+    else if (c["eos_token_id"].is_int())
+        spec.eos_token_ids.push_back(static_cast<int>(c["eos_token_id"].as_int()));
+    if (c["bos_token_id"].is_int()) spec.bos_token_id = static_cast<int>(c["bos_token_id"].as_int());
+    spec.validate();
+    return spec;
+}
+
+}  // namespace
+
 namespace {
 void register_builtin() {
     Architecture lfm2;
@@ -630,6 +835,13 @@ void register_builtin() {
     regipel.build_spec = regipel_build_spec;
     table()["Regipel"] = regipel;
     table()["regipel"] = regipel;
+    Architecture kifetar;
+    kifetar.name = "Kifetar";
+    kifetar.aliases = {"kifetar"};
+    kifetar.read_config = kifetar_read_config;
+    kifetar.build_spec = kifetar_build_spec;
+    table()["Kifetar"] = kifetar;
+    table()["kifetar"] = kifetar;
 }
 
 }  // namespace

@@ -10,6 +10,7 @@
 #include "../gemv_params.h"
 #include "../tile_params.h"
 #include "../no_alloc.h"
+#include "../norm_params.h"
 
 extern "C" {
 // elementwise.hip
@@ -141,4 +142,26 @@ int celeg_embed_stats(const void* table, const int* ids, float* out, float* stat
 int celeg_gemm_tiles_blocks(int M, int N, int K);
 int celeg_gemm_tiles_params_size();
 int celeg_gemm_tiles(const TileParams* params, int epi, hipStream_t stream);
+// norm_step.hip
+int celeg_norm_step(float* h, const void* y, int y_dtype, CelegNorm post, CelegNorm pre, void* out, int out_dtype,
+                    const int* rows, int n_rows, int width, int write_back, hipStream_t stream);
+int celeg_concat_rows(const float* a, const float* b, void* out, int out_dtype, int rows, int width, hipStream_t stream);
+// sigmoid_attention.hip
+int celeg_sigmoid_attention(const void* q, int ldq, const void* k_pool, const void* v_pool, int dtype, const int* table,
+                            int table_stride, const int* token_slot, const int* positions, const float* temp,
+                            const float* bias, const void* gate, int ldg, void* out, int ldo, int n_tokens, int q_heads,
+                            int kv_heads, int head_dim, int page_tokens, int n_layers, int layer, float scale, int window,
+                            hipStream_t stream);
+// delta_rule.hip
+int celeg_delta_prepare(const void* proj, int ld, int dtype, int col_b, int col_a, const float* conv_w, const float* a_log,
+                        const float* dt_bias, const float* conv_state, size_t state_stride, const int* positions,
+                        const int* token_seq, const int* seq_start, const int* token_slot, float* qk, float* v_out,
+                        float* beta_decay, int n_tokens, int G, int H, int D, int V, int taps, hipStream_t stream);
+int celeg_delta_conv_state(const void* proj, int ld, int dtype, float* conv_state, size_t state_stride, const int* cu_seqlens,
+                           const int* seq_slot, int n_seqs, int n_channels, int taps, hipStream_t stream);
+int celeg_delta_scan(const float* qk, const float* v, const float* beta_decay, float* state, size_t state_stride,
+                     const int* cu_seqlens, const int* seq_slot, float* out, int n_seqs, int G, int H, int D, int V,
+                     hipStream_t stream);
+int celeg_delta_gated_norm(const float* o, const float* w, const void* gate, int ldg, int dtype, float eps, void* out,
+                           int n_tokens, int H, int V, hipStream_t stream);
 }

@@ -14,6 +14,10 @@ namespace celeg {
 Model::Model(ModelSpec s) : spec(std::move(s)) {
     spec.validate();
     embedding_ = build_as<Embedding>("embedding", spec.embedding);
+    if (!spec.reinjection.kind.empty()) {
+        if (spec.streams != 1) throw SpecError("a reinjection of the embedding's rows works on one residual stream");
+        reinjection_ = build_as<Reinjection>("reinjection", spec.reinjection);
+    }
     for (const LayerSpec& layer : spec.layers) {
         blocks_.push_back(build_block(layer));
         if (blocks_.back()->streams() != spec.streams)
@@ -62,6 +66,7 @@ void Model::resolve_cache_sharing() {
 
 std::vector<std::pair<std::string, Part*>> Model::named_parts() {
     std::vector<std::pair<std::string, Part*>> out{{"embedding", embedding_.get()}};
+    if (reinjection_) out.emplace_back("reinjection", reinjection_.get());
     for (size_t i = 0; i < blocks_.size(); ++i)
         for (const auto& p : blocks_[i]->parts()) out.emplace_back("layers." + std::to_string(i) + "." + p.first, p.second);
     out.emplace_back("final_norm", final_norm_.get());
@@ -168,7 +173,21 @@ Tensor Model::forward(const StepBatch& batch, Runtime& rt) {
         hs = rt.ws.buf("hidden_streams", DType::F32, {T, S * width});
         rt.ops.streams_spread(h, hs, S);
     }
+    // the embedding's rows, kept for the entries of the run order that take them in again
+    Tensor x0;
+    if (reinjection_) {
+        x0 = rt.ws.buf("embedding_rows", DType::F32, {T, width});
+        rt.ops.cast(h, x0);
+    }
     for (size_t i = 0; i < spec.order.size(); ++i) {
+        if (spec.order[i].reinject) {
+            if (delta.defined()) rt.ops.norm_step(h, &delta, nullptr, nullptr, nullptr);     // the pending sum first
+            delta = Tensor();
+            rt.stream_stat_blocks = 0;
+            rt.stream_has_bf16 = false;
+            reinjection_->forward(h, x0, rt);
+            rt.mark("reinjection");
+        }
         delta = blocks_[static_cast<size_t>(spec.order[i].layer)]->forward(hs, delta, batch, caches_[i], rt);
         if (rt.after_layer) {
             if (S > 1) rt.ops.streams_sum(hs, h, S);

@@ -43,6 +43,7 @@ private:
     Mixer& mixer_of(int layer) { return blocks_[static_cast<size_t>(layer)]->mixer(); }
     void resolve_cache_sharing();
     std::unique_ptr<Embedding> embedding_;
+    std::unique_ptr<Reinjection> reinjection_;
     std::vector<std::unique_ptr<Block>> blocks_;
     std::unique_ptr<Norm> final_norm_;
     std::unique_ptr<Head> head_;

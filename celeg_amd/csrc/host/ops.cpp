@@ -51,6 +51,10 @@ const char* path_name(Path p) {
         case Path::AttentionDecodeFresh: return "attention_decode_fresh";
         case Path::AttentionRows: return "attention_rows";
         case Path::AttentionGeneral: return "attention_general";
+        case Path::AttentionSigmoid: return "attention_sigmoid";
+        case Path::AttentionSigmoidRows: return "attention_sigmoid_rows";
+        case Path::AttentionSigmoidDecode: return "attention_sigmoid_decode";
+        case Path::DeltaRule: return "delta_rule";
         case Path::AttentionLatent: return "attention_latent";
         case Path::AttentionLatentRows: return "attention_latent_rows";
         case Path::AttentionLatentDecode: return "attention_latent_decode";
@@ -375,6 +379,60 @@ void Ops::rmsnorm(const Tensor& x, const Tensor& weight, float eps, const Tensor
                                static_cast<int>(width), eps, write_back, stream), "rmsnorm");
 }
 
+// ---------------------------------------------------------------------------- norms as kernel arguments
+static CelegNorm norm_arg(const Ops::NormParams* p, long long width, const char* who) {
+    CelegNorm n{nullptr, nullptr, 0.f, CELEG_NORM_NONE};
+    if (!p) return n;
+    if (p->weight.defined()) {
+        dev(p->weight, "norm weight", DType::F32);
+        need(p->weight.numel() == width, std::string(who) + ": a norm weight must have the rows' width");
+        n.w = p->weight.as<float>();
+    }
+    if (p->bias.defined()) {
+        dev(p->bias, "norm bias", DType::F32);
+        need(p->bias.numel() == width, std::string(who) + ": a norm bias must have the rows' width");
+        n.b = p->bias.as<float>();
+    }
+    n.eps = p->eps;
+    n.mode = p->plain ? CELEG_NORM_NONE : p->centered ? CELEG_NORM_LAYER : CELEG_NORM_RMS;
+    return n;
+}
+
+void Ops::norm_step(const Tensor& h, const Tensor* y, const NormParams* post, const NormParams* pre, const Tensor* out,
+                    const int* rows) {
+    dev(h, "h", DType::F32);
+    need(h.ndim == 2, "norm_step: h must be a matrix");
+    const long long width = h.shape[1];
+    need(width * 4 <= 60 * 1024, "norm_step: rows of more than 15,360 values are not supported");
+    long long n_rows = h.shape[0];
+    if (y) {
+        dev(*y, "y");
+        need(y->ndim == 2 && y->shape[0] == h.shape[0] && y->shape[1] == width && y->contiguous(), "norm_step: y must have the shape of h");
+    }
+    if (out) {
+        dev(*out, "out");
+        need(out->ndim == 2 && out->shape[1] == width && out->contiguous(), "norm_step: out must have the width of h");
+        n_rows = out->shape[0];
+        need(rows || n_rows == h.shape[0], "norm_step: out must have the rows of h");
+        need(pre != nullptr, "norm_step: an output needs a norm");
+    }
+    need(!rows || out, "norm_step: a list of rows goes with an output");
+    need(y || out, "norm_step: nothing to do");
+    kernel_check(celeg_norm_step(h.as<float>(), y ? y->data : nullptr, y ? dt(*y, "y") : 0, norm_arg(y ? post : nullptr, width, "norm_step"),
+                                 norm_arg(pre, width, "norm_step"), out ? out->data : nullptr, out ? dt(*out, "out") : 0, rows,
+                                 static_cast<int>(n_rows), static_cast<int>(width), y && !rows ? 1 : 0, stream), "norm_step");
+}
+
+void Ops::concat_rows(const Tensor& a, const Tensor& b, const Tensor& out) {
+    dev(a, "a", DType::F32);
+    dev(b, "b", DType::F32);
+    dev(out, "out");
+    need(a.ndim == 2 && b.ndim == 2 && out.ndim == 2 && a.shape[0] == b.shape[0] && a.shape[1] == b.shape[1] &&
+             out.shape[0] == a.shape[0] && out.shape[1] == 2 * a.shape[1] && out.contiguous(), "concat_rows: shapes do not fit");
+    kernel_check(celeg_concat_rows(a.as<float>(), b.as<float>(), out.data, dt(out, "out"), static_cast<int>(a.shape[0]),
+                                   static_cast<int>(a.shape[1]), stream), "concat_rows");
+}
+
 void Ops::swiglu(const Tensor& gate_up, const Tensor& out) {
     dev(gate_up, "gate_up");
     dev(out, "out", gate_up.dtype);
@@ -678,6 +736,102 @@ void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_
                                        batch.positions, out.data, static_cast<int>(qw), static_cast<int>(T), heads,
                                        kv_heads, head_dim, kv.page_tokens, kv.n_layers, kv.layer, scale, window, stream),
                  "paged_attention");
+}
+
+// ---------------------------------------------------------------------------- attention with sigmoid weights
+void Ops::sigmoid_attention(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window,
+                            const Tensor* temp, const Tensor* bias, const Tensor* gate, const StepBatch& batch, const KVView& kv,
+                            Workspace&) {
+    dev(q, "q");
+    dev(out, "out", q.dtype);
+    const long long T = q.shape[0], qw = static_cast<long long>(heads) * head_dim;
+    need(q.ndim == 2 && out.ndim == 2 && T == batch.n_tokens && q.shape[1] == qw && out.shape[0] == T && out.shape[1] == qw &&
+             out.contiguous(), "sigmoid_attention: q and out must be [rows, heads*head_dim]");
+    need(head_dim <= 256, "sigmoid_attention: head_dim " + std::to_string(head_dim) + " exceeds 256");
+    need(heads % kv_heads == 0, "sigmoid_attention: heads must be a multiple of kv_heads");
+    check_kv(kv, kv_heads, head_dim, q.dtype);
+    for (const Tensor* per_head : {temp, bias})
+        if (per_head) {
+            dev(*per_head, "temperature / bias", DType::F32);
+            need(per_head->numel() == heads, "sigmoid_attention: one temperature and one bias per query head");
+        }
+    int ldg = 0;
+    if (gate) {
+        dev(*gate, "gate", q.dtype, false);
+        need(gate->ndim == 2 && gate->shape[0] == T && gate->shape[1] == heads, "sigmoid_attention: gate must be [rows, heads]");
+        ldg = rows_of(*gate, "gate");
+    }
+    took(Path::AttentionSigmoid);
+    kernel_check(celeg_sigmoid_attention(q.data, rows_of(q, "q"), kv.k, kv.v, dt(q, "q"), kv.table, kv.table_stride, batch.token_slot,
+                                         batch.positions, temp ? temp->as<float>() : nullptr, bias ? bias->as<float>() : nullptr,
+                                         gate ? gate->data : nullptr, ldg, out.data, static_cast<int>(qw), static_cast<int>(T), heads,
+                                         kv_heads, head_dim, kv.page_tokens, kv.n_layers, kv.layer, scale, window, stream),
+                 "sigmoid_attention");
+}
+
+// ---------------------------------------------------------------------------- gated delta rule
+void Ops::delta_prepare(const Tensor& proj, int col_b, int col_a, const DeltaShape& s, const Tensor& conv_w, const Tensor& a_log,
+                        const Tensor& dt_bias, const Tensor& conv_state, const Tensor& qk, const Tensor& v, const Tensor& beta_decay,
+                        const StepBatch& batch) {
+    dev(proj, "proj");
+    const long long T = proj.shape[0], qkw = 2LL * s.kv_heads * s.dim, vw = static_cast<long long>(s.heads) * s.vdim, C = qkw + vw;
+    need(s.heads > 0 && s.kv_heads > 0 && s.heads % s.kv_heads == 0 && s.dim > 0 && s.vdim > 0 && s.taps >= 1,
+         "delta_prepare: heads must be a positive multiple of kv_heads, sizes positive");
+    need(proj.ndim == 2 && T == batch.n_tokens && col_b >= C && col_a >= C && col_b + s.heads <= proj.shape[1] &&
+             col_a + s.heads <= proj.shape[1], "delta_prepare: the projections' columns do not fit");
+    dev(conv_w, "conv_w", DType::F32);
+    need(conv_w.numel() == C * s.taps, "delta_prepare: one row of taps per channel");
+    dev(a_log, "a_log", DType::F32);
+    dev(dt_bias, "dt_bias", DType::F32);
+    need(a_log.numel() == s.heads && dt_bias.numel() == s.heads, "delta_prepare: one decay constant and bias per head");
+    dev(conv_state, "conv_state", DType::F32, false);
+    need(conv_state.ndim == 3 && conv_state.shape[1] == std::max(s.taps - 1, 1) && conv_state.shape[2] == C &&
+             conv_state.stride[2] == 1 && conv_state.stride[1] == C, "delta_prepare: saved inputs must be [slots, taps - 1, channels]");
+    dev(qk, "qk", DType::F32);
+    dev(v, "v", DType::F32);
+    dev(beta_decay, "beta_decay", DType::F32);
+    need(qk.numel() == T * qkw && v.numel() == T * vw && beta_decay.numel() == T * 2 * s.heads, "delta_prepare: outputs do not fit");
+    const int ld = rows_of(proj, "proj");
+    took(Path::DeltaRule);
+    kernel_check(celeg_delta_prepare(proj.data, ld, dt(proj, "proj"), col_b, col_a, conv_w.as<float>(), a_log.as<float>(),
+                                     dt_bias.as<float>(), conv_state.as<float>(), static_cast<size_t>(conv_state.stride[0]),
+                                     batch.positions, batch.token_seq, batch.seq_start, batch.token_slot, qk.as<float>(), v.as<float>(),
+                                     beta_decay.as<float>(), static_cast<int>(T), s.kv_heads, s.heads, s.dim, s.vdim, s.taps, stream),
+                 "delta_prepare");
+    // (after every row has read the old saved inputs)
+    kernel_check(celeg_delta_conv_state(proj.data, ld, dt(proj, "proj"), conv_state.as<float>(), static_cast<size_t>(conv_state.stride[0]),
+                                        batch.cu_seqlens, batch.seq_slot, batch.n_seqs, static_cast<int>(C), s.taps, stream),
+                 "delta_conv_state");
+}
+
+void Ops::delta_scan(const Tensor& qk, const Tensor& v, const Tensor& beta_decay, const Tensor& state, const Tensor& out,
+                     const DeltaShape& s, const StepBatch& batch) {
+    dev(qk, "qk", DType::F32);
+    dev(v, "v", DType::F32);
+    dev(beta_decay, "beta_decay", DType::F32);
+    dev(out, "out", DType::F32);
+    dev(state, "state", DType::F32, false);
+    const long long T = batch.n_tokens, per_slot = static_cast<long long>(s.heads) * s.dim * s.vdim;
+    need(qk.numel() == T * 2 * s.kv_heads * s.dim && v.numel() == T * s.heads * s.vdim && out.numel() == v.numel() &&
+             beta_decay.numel() == T * 2 * s.heads, "delta_scan: rows do not fit");
+    need(state.ndim >= 2 && state.numel() / state.shape[0] == per_slot && state.stride[state.ndim - 1] == 1,
+         "delta_scan: state must be [slots, heads, dim, vdim]");
+    need((static_cast<long long>(s.dim) * 64 + 2 * s.dim) * 4 <= 64 * 1024, "delta_scan: dim " + std::to_string(s.dim) + " exceeds 248");
+    kernel_check(celeg_delta_scan(qk.as<float>(), v.as<float>(), beta_decay.as<float>(), state.as<float>(),
+                                  static_cast<size_t>(state.stride[0]), batch.cu_seqlens, batch.seq_slot, out.as<float>(), batch.n_seqs,
+                                  s.kv_heads, s.heads, s.dim, s.vdim, stream), "delta_scan");
+}
+
+void Ops::delta_gated_norm(const Tensor& o, const Tensor& weight, const Tensor& gate, float eps, const Tensor& out, int heads, int vdim) {
+    dev(o, "o", DType::F32);
+    dev(weight, "weight", DType::F32);
+    dev(gate, "gate", out.dtype, false);
+    dev(out, "out");
+    const long long T = o.shape[0], w = static_cast<long long>(heads) * vdim;
+    need(o.ndim == 2 && o.shape[1] == w && out.ndim == 2 && out.shape[0] == T && out.shape[1] == w && out.contiguous() &&
+             gate.ndim == 2 && gate.shape[0] == T && gate.shape[1] == w && weight.numel() == vdim, "delta_gated_norm: shapes do not fit");
+    kernel_check(celeg_delta_gated_norm(o.as<float>(), weight.as<float>(), gate.data, rows_of(gate, "gate"), dt(out, "out"), eps, out.data,
+                                        static_cast<int>(T), heads, vdim, stream), "delta_gated_norm");
 }
 
 // Where the context of few requests is cut into parts: how many wavefronts a part's workgroup has

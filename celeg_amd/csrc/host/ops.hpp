@@ -102,7 +102,7 @@ struct StepPrologue {
 // graph records; a replay counts nothing): what tests and tools ask to see that a size took the
 // path it was meant to take.
 enum class Path : int {
-    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, AttentionLatent, AttentionLatentRows, AttentionLatentDecode, RoutedExperts, LinearF32, LinearLibrary, LinearStandIn,
+    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, AttentionSigmoid, AttentionSigmoidRows, AttentionSigmoidDecode, DeltaRule, AttentionLatent, AttentionLatentRows, AttentionLatentDecode, RoutedExperts, LinearF32, LinearLibrary, LinearStandIn,
     FusedSliced, FusedRows, FusedStaged, Tiled, TiledQkv, ArgmaxMerged, Count
 };
 const char* path_name(Path p);
@@ -148,6 +148,21 @@ public:
                     const Tensor* in_w, const Tensor* weight, float eps, const Tensor* normed);
     void rmsnorm(const Tensor& x, const Tensor& weight, float eps, const Tensor& out, const Tensor* delta = nullptr,
                  const int* rows = nullptr);
+    // What a norm does to a row, for kernels that take a norm as an argument: weight and bias
+    // (32-bit, either may be undefined), eps, and whether the mean is taken off first (a layer
+    // norm) or not (an RMS norm); `plain`: no normalisation at all.
+    struct NormParams {
+        Tensor weight, bias;
+        float eps = 0.f;
+        bool centered = false, plain = false;
+    };
+    // One sub-layer boundary on a single 32-bit stream h [rows, width]: if y is given,
+    // h += post(y) (post null: the plain sum); then, if out is given, out = pre(h).  With `rows`
+    // only those rows of h are read, nothing is written back, and out has one row per entry.
+    void norm_step(const Tensor& h, const Tensor* y, const NormParams* post, const NormParams* pre, const Tensor* out,
+                   const int* rows = nullptr);
+    // out [rows, 2 * width] = (a | b), both 32-bit [rows, width]
+    void concat_rows(const Tensor& a, const Tensor& b, const Tensor& out);
     void swiglu(const Tensor& gate_up, const Tensor& out);
     void add_bias(const Tensor& x, const Tensor& bias);
     void cast(const Tensor& src, const Tensor& dst);
@@ -165,6 +180,25 @@ public:
                             int kv_heads, int head_dim, const StepBatch& batch, const KVView& kv);
     void paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
                          int window, const StepBatch& batch, const KVView& kv, Workspace& ws, const FreshKV* fresh = nullptr);
+    // Attention with sigmoid weights: weight = sigmoid((q . k) * scale * temp[h] + bias[h]), not
+    // normalised over the keys; temp and bias [heads] 32-bit or null; gate: raw gate values, the
+    // head's result is multiplied by sigmoid(gate[row, h]) (a view [rows, heads] with dense rows, or null).
+    void sigmoid_attention(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale, int window,
+                           const Tensor* temp, const Tensor* bias, const Tensor* gate, const StepBatch& batch, const KVView& kv,
+                           Workspace& ws);
+    // The gated delta rule.  heads value heads of vdim, kv_heads query/key heads of dim.
+    struct DeltaShape { int heads = 0, kv_heads = 0, dim = 0, vdim = 0, taps = 0; };
+    // proj [rows, >= col_a + heads]: q | k | v channels from column 0, write strengths at col_b, decay inputs
+    // at col_a.  Leaves qk [rows, 2 * kv_heads * dim] (unit keys, scaled unit queries), v [rows, heads * vdim]
+    // and beta_decay [rows, 2 * heads], all 32-bit, and moves the requests' saved inputs on.
+    void delta_prepare(const Tensor& proj, int col_b, int col_a, const DeltaShape& shape, const Tensor& conv_w, const Tensor& a_log,
+                       const Tensor& dt_bias, const Tensor& conv_state, const Tensor& qk, const Tensor& v, const Tensor& beta_decay,
+                       const StepBatch& batch);
+    // the recurrence over the step's rows of every request, from and into state [slots, heads, dim, vdim]
+    void delta_scan(const Tensor& qk, const Tensor& v, const Tensor& beta_decay, const Tensor& state, const Tensor& out,
+                    const DeltaShape& shape, const StepBatch& batch);
+    // out = o / rms(o) * weight * silu(gate) per head; o [rows, heads * vdim] 32-bit, gate a view with dense rows
+    void delta_gated_norm(const Tensor& o, const Tensor& weight, const Tensor& gate, float eps, const Tensor& out, int heads, int vdim);
     // whether a decode-only step's attention can prepare and write the step's own keys and values itself
     bool attention_fresh_ok(int heads, int head_dim, const Tensor* inv_freq, int rotary_dim, int pairing, const StepBatch& batch,
                             const KVView& kv, DType dtype) const;

@@ -18,7 +18,7 @@ namespace celeg {
 namespace {
 struct Registries {
     std::map<std::string, std::map<std::string, PartFactory>> parts{
-        {"norm", {}}, {"mixer", {}}, {"ffn", {}}, {"position", {}}, {"embedding", {}}, {"head", {}}, {"link", {}}};
+        {"norm", {}}, {"mixer", {}}, {"ffn", {}}, {"position", {}}, {"embedding", {}}, {"head", {}}, {"link", {}}, {"reinjection", {}}};
     std::map<std::string, BlockFactory> blocks;
     std::mutex lock;
 };
@@ -142,7 +142,10 @@ public:
             weight_ = from_host_floats(w, DType::F32, {width_});
         }
         foldable_ = Foldable{weight_->view, static_cast<float>(eps_)};
+        params_.weight = weight_->view;
+        params_.eps = static_cast<float>(eps_);
     }
+    const Ops::NormParams* params() const override { return weight_ ? &params_ : nullptr; }
     void forward(const Tensor& x, const Tensor& out, Runtime& rt, const Tensor* delta, const int* rows) override {
         rt.ops.rmsnorm(x, weight_->view, static_cast<float>(eps_), out, delta, rows);
     }
@@ -153,6 +156,7 @@ private:
     double eps_, offset_;
     std::shared_ptr<DeviceTensor> weight_;
     Foldable foldable_;
+    Ops::NormParams params_;
 };
 
 // y = x (+ delta): no normalisation, no weight.  With it a test sees a part's rows as they are.
@@ -215,20 +219,44 @@ public:
         const std::string pairing = s.params.get_string("pairing", "halves");
         if (pairing != "halves" && pairing != "neighbours") throw SpecError("rope: pairing is 'halves' or 'neighbours', not '" + pairing + "'");
         pairing_ = pairing == "neighbours" ? 1 : 0;
+        if (!s.params["scaling"].is_null()) {
+            const Json& sc = s.params["scaling"];
+            if (!sc.is_object()) throw SpecError("rope: scaling must be an object");
+            scaled_ = true;
+            factor_ = sc.get_double("factor", 1.0);
+            low_ = sc.get_double("low", 1.0);
+            high_ = sc.get_double("high", 1.0);
+            original_ = sc.get_double("original", 0.0);
+            if (!(factor_ > 0) || !(low_ > 0) || !(high_ > low_) || !(original_ > 0))
+                throw SpecError("rope: scaling needs factor > 0, 0 < low < high and original > 0");
+        }
     }
     bool graph_safe() const override { return true; }
     Tables tables(Runtime&) override {
         if (!table_) {
             std::vector<float> freq(static_cast<size_t>(rotary_dim_ / 2));
             for (int i = 0; i < rotary_dim_ / 2; ++i)
-                freq[static_cast<size_t>(i)] = static_cast<float>(std::pow(theta_, -2.0 * i / rotary_dim_));
+                freq[static_cast<size_t>(i)] = static_cast<float>(scaled(std::pow(theta_, -2.0 * i / rotary_dim_)));
             table_ = from_host_floats(freq, DType::F32, {rotary_dim_ / 2});
         }
         return Tables{table_->view, rotary_dim_, pairing_};
     }
 
 private:
+    // "scaling" {factor, low, high, original}: frequencies whose wavelength 2 pi / f is below
+    // original / high stay, above original / low become f / factor, and between the two
+    // (1 - s) f / factor + s f with s = (original / wavelength - low) / (high - low)
+    double scaled(double f) const {
+        if (!scaled_) return f;
+        const double wavelength = 2.0 * 3.14159265358979323846 / f;
+        if (wavelength < original_ / high_) return f;
+        if (wavelength > original_ / low_) return f / factor_;
+        const double t = (original_ / wavelength - low_) / (high_ - low_);
+        return (1.0 - t) * f / factor_ + t * f;
+    }
     double theta_;
+    bool scaled_ = false;
+    double factor_ = 1.0, low_ = 1.0, high_ = 1.0, original_ = 0.0;
     int head_dim_, rotary_dim_, pairing_ = 0;
     std::shared_ptr<DeviceTensor> table_;
 };
@@ -1058,6 +1086,340 @@ private:
     std::unique_ptr<HyperLink> ffn_link_;
 };
 
+// ---------------------------------------------------------------------------- layer norm
+// y = (x - mean) / sqrt(var + eps) * w + b, var the mean of the squared deviations from the
+// mean, eps inside the root; statistics and scaling in 32-bit.  "bias": false leaves b out.
+class LayerNorm final : public Norm {
+public:
+    explicit LayerNorm(const PartSpec& s)
+        : Norm(s), width_(s.params.get_int("width", 0)), eps_(s.params.get_double("eps", 0.0)), bias_(s.params.get_bool("bias", true)) {
+        if (width_ <= 0 || !(eps_ > 0)) throw SpecError("layernorm: width and eps must be positive");
+    }
+    bool graph_safe() const override { return true; }
+    WeightSpecs weight_specs() const override {
+        WeightSpecs specs{{"weight", vec(width_, "around_one")}};
+        if (bias_) specs.push_back({"bias", vec(width_)});
+        return specs;
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        weight_ = get(t, "weight");
+        if (bias_) b_ = get(t, "bias");
+        params_.weight = weight_->view;
+        if (b_) params_.bias = b_->view;
+        params_.eps = static_cast<float>(eps_);
+        params_.centered = true;
+    }
+    void forward(const Tensor& x, const Tensor& out, Runtime& rt, const Tensor* delta, const int* rows) override {
+        if (x.dtype != DType::F32) throw SpecError("layernorm: the rows to normalise must be 32-bit");
+        rt.ops.norm_step(x, delta, nullptr, &params_, &out, rows);
+    }
+    const Ops::NormParams* params() const override { return weight_ ? &params_ : nullptr; }
+
+private:
+    long long width_;
+    double eps_;
+    bool bias_;
+    std::shared_ptr<DeviceTensor> weight_, b_;
+    Ops::NormParams params_;
+};
+
+// ---------------------------------------------------------------------------- attention with sigmoid weights
+// Grouped-query attention whose weights are sigmoids of the scores instead of a softmax over them.
+//
+// q = W_q h (+ b_q), k = W_k h (+ b_k); the values are the keys as projected, before norm and
+// rotation ("values": "keys"; there is then no value projection), or v = W_v h ("values":
+// "projected").  RMS norm of every q and k head over head_dim with one weight for all heads
+// ("qk_norm"), then the position encoding of q and k.  The weight of key j for query i of head
+// h, j inside the window [i - window + 1, i] (or all j <= i without one), is
+//     sigmoid((q_i . k_j) * scale * temp[h] + pb[h])
+// ("temperature" and "score_bias": a learned number per head each), not normalised over the
+// keys.  With "head_gate" the head's result is multiplied by sigmoid(W_g h)[h], one number per
+// head from the mixer's own input.  The heads, side by side, go through W_o.
+class SigmoidAttention final : public Mixer {
+public:
+    explicit SigmoidAttention(const PartSpec& s) : Mixer(s) {
+        const Json& p = s.params;
+        width_ = p.get_int("width", 0);
+        heads_ = static_cast<int>(p.get_int("heads", 0));
+        kv_heads_ = static_cast<int>(p.get_int("kv_heads", heads_));
+        head_dim_ = static_cast<int>(p.get_int("head_dim", 0));
+        qk_norm_ = p.get_bool("qk_norm", false);
+        bias_ = p.get_bool("bias", false);
+        temperature_ = p.get_bool("temperature", false);
+        score_bias_ = p.get_bool("score_bias", false);
+        head_gate_ = p.get_bool("head_gate", false);
+        eps_ = static_cast<float>(p.get_double("eps", 1e-6));
+        const std::string values = p.get_string("values", "projected");
+        if (values != "keys" && values != "projected") throw SpecError("sigmoid_attention: values is 'keys' or 'projected', not '" + values + "'");
+        values_are_keys_ = values == "keys";
+        if (!p["window"].is_null()) {
+            window_ = static_cast<int>(p["window"].as_int());
+            if (*window_ <= 0) throw SpecError("sigmoid_attention: window must be positive");
+        }
+        if (width_ <= 0 || heads_ <= 0 || kv_heads_ <= 0 || heads_ % kv_heads_)
+            throw SpecError("sigmoid_attention: heads must be a positive multiple of kv_heads");
+        if (head_dim_ <= 0 || head_dim_ % 2) throw SpecError("sigmoid_attention: head_dim must be even");
+        scale_ = p["scale"].is_null() ? static_cast<float>(1.0 / std::sqrt(static_cast<double>(head_dim_)))
+                                      : static_cast<float>(p["scale"].as_double());
+        PartSpec none;
+        none.kind = "none";
+        position_ = build_as<PositionEncoding>(
+            "position", PartSpec::is_part(p["position"]) ? PartSpec::from_json(p["position"], "sigmoid_attention.position") : none);
+    }
+    bool graph_safe() const override { return true; }
+    std::vector<const Part*> children() const override { return {position_.get()}; }
+    std::optional<KVNeed> kv_need() const override { return KVNeed{kv_heads_, head_dim_, window_}; }
+    WeightSpecs weight_specs() const override {
+        const long long qw = static_cast<long long>(heads_) * head_dim_, kvw = static_cast<long long>(kv_heads_) * head_dim_;
+        WeightSpecs specs{{"q", matrix(qw, width_)}, {"k", matrix(kvw, width_)}, {"o", matrix(width_, qw)}};
+        if (!values_are_keys_) specs.push_back({"v", matrix(kvw, width_)});
+        if (bias_) {
+            specs.push_back({"q_bias", vec(qw)});
+            specs.push_back({"k_bias", vec(kvw)});
+        }
+        if (qk_norm_) {
+            specs.push_back({"q_norm", vec(head_dim_, "around_one")});
+            specs.push_back({"k_norm", vec(head_dim_, "around_one")});
+        }
+        if (temperature_) specs.push_back({"temp", vec(heads_, "around_one")});
+        if (score_bias_) specs.push_back({"pb", vec(heads_)});
+        if (head_gate_) specs.push_back({"g", matrix(heads_, width_)});
+        return specs;
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        // every projection of the mixer's input in one product; the gate's few rows are padded with
+        // zero rows to a multiple of 16 columns
+        const long long qw = static_cast<long long>(heads_) * head_dim_, kvw = static_cast<long long>(kv_heads_) * head_dim_;
+        std::vector<std::shared_ptr<DeviceTensor>> in{get(t, "q"), get(t, "k")};
+        if (!values_are_keys_) in.push_back(get(t, "v"));
+        gate_col_ = qw + kvw * (values_are_keys_ ? 1 : 2);
+        long long cols = gate_col_;
+        if (head_gate_) {
+            in.push_back(get(t, "g"));
+            const long long pad = (16 - heads_ % 16) % 16;
+            if (pad) in.push_back(from_host_floats(std::vector<float>(static_cast<size_t>(pad * width_), 0.f), in[0]->view.dtype, {pad, width_}));
+            cols += heads_ + pad;
+        }
+        for (const auto& w : in)
+            if (w->view.dtype != in[0]->view.dtype) throw SpecError("sigmoid_attention: the input projections are stored in different dtypes");
+        w_in_ = concat_rows(in);
+        if (bias_) {
+            std::vector<float> b = to_host_floats(get(t, "q_bias")->view), kb = to_host_floats(get(t, "k_bias")->view);
+            b.insert(b.end(), kb.begin(), kb.end());
+            b.resize(static_cast<size_t>(cols), 0.f);
+            b_in_ = from_host_floats(b, DType::F32, {cols});
+        }
+        w_o_ = get(t, "o");
+        q_norm_ = maybe(t, "q_norm");
+        k_norm_ = maybe(t, "k_norm");
+        temp_ = maybe(t, "temp");
+        pb_ = maybe(t, "pb");
+    }
+    Tensor forward(const Tensor& x, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
+        if (!cache.kv) throw SpecError("sigmoid_attention: the cache has no keys and values for this layer");
+        if (!cache.writes_kv) throw SpecError("sigmoid_attention: reading another entry's cache is not supported");
+        const long long T = x.shape[0];
+        const long long qw = static_cast<long long>(heads_) * head_dim_, kvw = static_cast<long long>(kv_heads_) * head_dim_;
+        Tensor proj = rt.ws.buf("sattn_proj", rt.dtype, {T, w_in_->view.shape[0]});
+        rt.ops.linear(x, w_in_->view, proj, b_in_ ? &b_in_->view : nullptr, rt.ws);
+        Tensor q = proj.cols(0, qw), k = proj.cols(qw, kvw);
+        Tensor v = values_are_keys_ ? k : proj.cols(qw + kvw, kvw);
+        Tensor gate = head_gate_ ? proj.cols(gate_col_, heads_) : Tensor();
+        const PositionEncoding::Tables tables = position_->tables(rt);
+        const Tensor* inv_freq = tables.inv_freq.defined() ? &tables.inv_freq : nullptr;
+        // (q is normed and turned in place; the keys go to their pages normed and turned, the values as they are)
+        rt.ops.qk_norm_rope_store(q, &k, &v, q_norm_ ? &q_norm_->view : nullptr, k_norm_ ? &k_norm_->view : nullptr, eps_, inv_freq,
+                                  tables.rotary_dim, tables.pairing, heads_, kv_heads_, head_dim_, batch, *cache.kv);
+        Tensor attended = rt.ws.buf("sattn_out", rt.dtype, {T, qw});
+        rt.ops.sigmoid_attention(q, attended, heads_, kv_heads_, head_dim_, scale_, window_ ? *window_ : 0,
+                                 temp_ ? &temp_->view : nullptr, pb_ ? &pb_->view : nullptr, head_gate_ ? &gate : nullptr, batch,
+                                 *cache.kv, rt.ws);
+        Tensor out = rt.ws.buf("mixer_out", rt.dtype, {T, width_});
+        rt.ops.linear(attended, w_o_->view, out, nullptr, rt.ws);
+        return out;
+    }
+
+private:
+    long long width_ = 0, gate_col_ = 0;
+    int heads_ = 0, kv_heads_ = 0, head_dim_ = 0;
+    bool qk_norm_ = false, bias_ = false, temperature_ = false, score_bias_ = false, head_gate_ = false, values_are_keys_ = false;
+    float eps_ = 1e-6f, scale_ = 1.f;
+    std::optional<int> window_;
+    std::unique_ptr<PositionEncoding> position_;
+    std::shared_ptr<DeviceTensor> w_in_, b_in_, w_o_, q_norm_, k_norm_, temp_, pb_;
+};
+
+// ---------------------------------------------------------------------------- gated delta rule
+// A recurrent mixer with a matrix of state per head.
+//
+// q = W_q h and k = W_k h (kv_heads heads of dim), v = W_v h (heads of vdim; value head i uses
+// query/key head i / (heads / kv_heads)); each channel of q, k and v passes a short causal
+// convolution over time (taps [channels, taps], the last tap the current token's, zeros before
+// the sequence starts) and silu; q and k become unit vectors per head
+// (x / sqrt(sum x^2 + 1e-6)), q times dim^-1/2.  beta = sigmoid(W_b h) and the decay
+// a = exp(-exp(A_log) softplus(W_a h + dt_bias)), one each per value head.  Per head and token
+//     S <- a S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+// so the read-out sees the token's own write.  o is RMS-normed per head over vdim (weight
+// [vdim] shared by the heads) and multiplied by silu(W_g h); the heads go through W_o.
+//
+// State per request: S [heads, dim, vdim] and the last taps - 1 inputs of the convolutions
+// [taps - 1, channels], both 32-bit.  Everything from the convolutions' sums to the gated norm
+// is 32-bit in both dtypes.
+class GatedDeltaRule final : public Mixer {
+public:
+    explicit GatedDeltaRule(const PartSpec& s) : Mixer(s) {
+        const Json& p = s.params;
+        width_ = p.get_int("width", 0);
+        shape_.heads = static_cast<int>(p.get_int("heads", 0));
+        shape_.kv_heads = static_cast<int>(p.get_int("kv_heads", shape_.heads));
+        shape_.dim = static_cast<int>(p.get_int("dim", 0));
+        shape_.vdim = static_cast<int>(p.get_int("vdim", shape_.dim));
+        shape_.taps = static_cast<int>(p.get_int("taps", 0));
+        eps_ = static_cast<float>(p.get_double("eps", 1e-6));
+        if (width_ <= 0 || shape_.heads <= 0 || shape_.kv_heads <= 0 || shape_.heads % shape_.kv_heads)
+            throw SpecError("gated_delta_rule: heads must be a positive multiple of kv_heads");
+        if (shape_.dim <= 0 || shape_.vdim <= 0 || shape_.taps <= 0) throw SpecError("gated_delta_rule: dim, vdim and taps must be positive");
+    }
+    bool graph_safe() const override { return true; }
+    long long qk_width() const { return static_cast<long long>(shape_.kv_heads) * shape_.dim; }
+    long long v_width() const { return static_cast<long long>(shape_.heads) * shape_.vdim; }
+    long long channels() const { return 2 * qk_width() + v_width(); }
+    std::vector<StateNeed> state_needs() const override {
+        return {StateNeed{"S", {shape_.heads, shape_.dim, shape_.vdim}, DType::F32},
+                StateNeed{"conv", {std::max(shape_.taps - 1, 1), channels()}, DType::F32}};
+    }
+    WeightSpecs weight_specs() const override {
+        auto taps = [&](long long n) { return WeightSpec{{n, shape_.taps}, "vector", "normal", {}}; };
+        return {{"q", matrix(qk_width(), width_)}, {"k", matrix(qk_width(), width_)}, {"v", matrix(v_width(), width_)},
+                {"q_conv", taps(qk_width())},      {"k_conv", taps(qk_width())},      {"v_conv", taps(v_width())},
+                {"b", matrix(shape_.heads, width_)}, {"a", matrix(shape_.heads, width_)}, {"A_log", vec(shape_.heads)},
+                {"dt_bias", vec(shape_.heads)},    {"norm", vec(shape_.vdim, "around_one")}, {"g", matrix(v_width(), width_)},
+                {"o", matrix(width_, v_width())}};
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        // one product for everything that reads the mixer's input: q | k | v | gate | b | a (| zero rows)
+        std::vector<std::shared_ptr<DeviceTensor>> in{get(t, "q"), get(t, "k"), get(t, "v"), get(t, "g"), get(t, "b"), get(t, "a")};
+        for (const auto& w : in)
+            if (w->view.dtype != in[0]->view.dtype) throw SpecError("gated_delta_rule: the input projections are stored in different dtypes");
+        col_gate_ = channels();
+        col_b_ = col_gate_ + v_width();
+        col_a_ = col_b_ + shape_.heads;
+        const long long cols = col_a_ + shape_.heads, pad = (16 - cols % 16) % 16;
+        if (pad) in.push_back(from_host_floats(std::vector<float>(static_cast<size_t>(pad * width_), 0.f), in[0]->view.dtype, {pad, width_}));
+        w_in_ = concat_rows(in);
+        conv_w_ = concat_rows({get(t, "q_conv"), get(t, "k_conv"), get(t, "v_conv")});
+        a_log_ = get(t, "A_log");
+        dt_bias_ = get(t, "dt_bias");
+        norm_ = get(t, "norm");
+        w_o_ = get(t, "o");
+    }
+    Tensor forward(const Tensor& x, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
+        const long long T = x.shape[0];
+        Tensor proj = rt.ws.buf("delta_proj", rt.dtype, {T, w_in_->view.shape[0]});
+        rt.ops.linear(x, w_in_->view, proj, nullptr, rt.ws);
+        Tensor qk = rt.ws.buf("delta_qk", DType::F32, {T, 2 * qk_width()});
+        Tensor v = rt.ws.buf("delta_v", DType::F32, {T, v_width()});
+        Tensor beta_decay = rt.ws.buf("delta_beta_decay", DType::F32, {T, 2LL * shape_.heads});
+        rt.ops.delta_prepare(proj, static_cast<int>(col_b_), static_cast<int>(col_a_), shape_, conv_w_->view, a_log_->view,
+                             dt_bias_->view, cache.states.at("conv"), qk, v, beta_decay, batch);
+        Tensor o = rt.ws.buf("delta_o", DType::F32, {T, v_width()});
+        rt.ops.delta_scan(qk, v, beta_decay, cache.states.at("S"), o, shape_, batch);
+        Tensor gated = rt.ws.buf("delta_gated", rt.dtype, {T, v_width()});
+        rt.ops.delta_gated_norm(o, norm_->view, proj.cols(col_gate_, v_width()), eps_, gated, shape_.heads, shape_.vdim);
+        Tensor out = rt.ws.buf("mixer_out", rt.dtype, {T, width_});
+        rt.ops.linear(gated, w_o_->view, out, nullptr, rt.ws);
+        return out;
+    }
+
+private:
+    long long width_ = 0, col_gate_ = 0, col_b_ = 0, col_a_ = 0;
+    Ops::DeltaShape shape_;
+    float eps_ = 1e-6f;
+    std::shared_ptr<DeviceTensor> w_in_, conv_w_, a_log_, dt_bias_, norm_, w_o_;
+};
+
+// ---------------------------------------------------------------------------- the embedding's rows, again
+// linear_concat: h <- W [h ; x0], W [width, 2 * width] with the stream's columns first.
+class LinearReinjection final : public Reinjection {
+public:
+    explicit LinearReinjection(const PartSpec& s) : Reinjection(s), width_(s.params.get_int("width", 0)) {
+        if (width_ <= 0) throw SpecError("linear_concat: width must be positive");
+    }
+    bool graph_safe() const override { return true; }
+    WeightSpecs weight_specs() const override { return {{"weight", matrix(width_, 2 * width_)}}; }
+    void load(const PartTensors& t, Runtime&) override { weight_ = get(t, "weight"); }
+    void forward(const Tensor& h, const Tensor& x0, Runtime& rt) override {
+        const long long T = h.shape[0];
+        Tensor both = rt.ws.buf("reinjection_in", rt.dtype, {T, 2 * width_});
+        rt.ops.concat_rows(h, x0, both);
+        rt.ops.linear(both, weight_->view, h, nullptr, rt.ws);      // (h was copied: the product may write it)
+    }
+
+private:
+    long long width_;
+    std::shared_ptr<DeviceTensor> weight_;
+};
+
+// ---------------------------------------------------------------------------- norms before and after
+// sandwich_norm: h += post1(mixer(pre1(h))); h += post2(ffn(pre2(h))).  The stream is 32-bit
+// and so are the norms' statistics and the sums.  One kernel per boundary: the first norms the
+// stream, the second adds the mixer's normed output and norms for the feed-forward, the third
+// adds the feed-forward's normed output.  A feed-forward of kind "none" is left out with its norms.
+class SandwichBlock final : public Block {
+public:
+    explicit SandwichBlock(const LayerSpec& layer)
+        : mixer_norm_(build_as<Norm>("norm", layer.mixer_norm)), mixer_(build_as<Mixer>("mixer", layer.mixer)),
+          mixer_post_(build_as<Norm>("norm", layer.mixer_post_norm)), has_ffn_(layer.ffn.kind != "none") {
+        if (has_ffn_) {
+            ffn_norm_ = build_as<Norm>("norm", layer.ffn_norm);
+            ffn_ = build_as<FeedForward>("ffn", layer.ffn);
+            ffn_post_ = build_as<Norm>("norm", layer.ffn_post_norm);
+        }
+    }
+    std::vector<std::pair<std::string, Part*>> parts() override {
+        std::vector<std::pair<std::string, Part*>> out{{"mixer_norm", mixer_norm_.get()}, {"mixer", mixer_.get()}, {"mixer_post_norm", mixer_post_.get()}};
+        if (has_ffn_) {
+            out.emplace_back("ffn_norm", ffn_norm_.get());
+            out.emplace_back("ffn", ffn_.get());
+            out.emplace_back("ffn_post_norm", ffn_post_.get());
+        }
+        return out;
+    }
+    Mixer& mixer() override { return *mixer_; }
+    Tensor forward(const Tensor& h, const Tensor& delta, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
+        const long long T = h.shape[0], width = h.shape[1];
+        rt.stream_stat_blocks = 0;
+        rt.stream_has_bf16 = false;
+        Tensor normed = rt.ws.buf("normed", rt.dtype, {T, width});
+        rt.ops.norm_step(h, delta.defined() ? &delta : nullptr, nullptr, &of(*mixer_norm_), &normed);
+        Tensor y = mixer_->forward(normed, batch, cache, rt);
+        rt.mark("mixer " + mixer_->spec.kind);
+        if (!has_ffn_) {
+            rt.ops.norm_step(h, &y, &of(*mixer_post_), nullptr, nullptr);
+            return Tensor();
+        }
+        rt.ops.norm_step(h, &y, &of(*mixer_post_), &of(*ffn_norm_), &normed);
+        y = ffn_->forward(normed, batch, rt);
+        rt.ops.norm_step(h, &y, &of(*ffn_post_), nullptr, nullptr);
+        rt.mark("ffn " + ffn_->spec.kind);
+        return Tensor();
+    }
+
+private:
+    static const Ops::NormParams& of(const Norm& norm) {
+        const Ops::NormParams* p = norm.params();
+        if (!p) throw SpecError("sandwich_norm: norm '" + norm.spec.kind + "' cannot be taken into the boundary kernels");
+        return *p;
+    }
+    std::unique_ptr<Norm> mixer_norm_;
+    std::unique_ptr<Mixer> mixer_;
+    std::unique_ptr<Norm> mixer_post_;
+    bool has_ffn_;
+    std::unique_ptr<Norm> ffn_norm_;
+    std::unique_ptr<FeedForward> ffn_;
+    std::unique_ptr<Norm> ffn_post_;
+};
+
 template <typename T>
 PartFactory factory_of() {
     return [](const PartSpec& s) { return std::unique_ptr<Part>(new T(s)); };
@@ -1068,11 +1430,15 @@ void register_builtin_parts() {
     std::lock_guard<std::mutex> guard(r.lock);
     r.parts["norm"]["rmsnorm"] = factory_of<RmsNorm>();
     r.parts["norm"]["identity"] = factory_of<IdentityNorm>();
+    r.parts["norm"]["layernorm"] = factory_of<LayerNorm>();
     r.parts["position"]["rope"] = factory_of<Rope>();
     r.parts["position"]["none"] = factory_of<NoPosition>();
     r.parts["mixer"]["gqa_attention"] = factory_of<GqaAttention>();
     r.parts["mixer"]["latent_attention"] = factory_of<LatentAttention>();
     r.parts["mixer"]["short_conv"] = factory_of<ShortConv>();
+    r.parts["mixer"]["sigmoid_attention"] = factory_of<SigmoidAttention>();
+    r.parts["mixer"]["gated_delta_rule"] = factory_of<GatedDeltaRule>();
+    r.parts["reinjection"]["linear_concat"] = factory_of<LinearReinjection>();
     r.parts["mixer"]["none"] = factory_of<NoMixer>();
     r.parts["ffn"]["swiglu"] = factory_of<SwiGlu>();
     r.parts["ffn"]["routed_experts"] = factory_of<RoutedExperts>();
@@ -1083,6 +1449,7 @@ void register_builtin_parts() {
     r.parts["head"]["linear_head"] = factory_of<LinearHead>();
     r.parts["head"]["hidden"] = factory_of<HiddenHead>();
     r.blocks["pre_norm"] = [](const LayerSpec& layer) { return std::unique_ptr<Block>(new PreNormBlock(layer)); };
+    r.blocks["sandwich_norm"] = [](const LayerSpec& layer) { return std::unique_ptr<Block>(new SandwichBlock(layer)); };
     r.blocks["hyper_connections"] = [](const LayerSpec& layer) { return std::unique_ptr<Block>(new HyperBlock(layer)); };
 }
 

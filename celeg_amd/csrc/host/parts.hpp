@@ -62,6 +62,17 @@ public:
     // rows' 1/rms); nullptr otherwise.
     struct Foldable { Tensor weight; float eps; };
     virtual const Foldable* foldable() const { return nullptr; }
+    // What the norm does to a row, if that is a scale and a bias around a normalisation that a
+    // kernel with a norm among its arguments can do itself; nullptr otherwise.
+    virtual const Ops::NormParams* params() const { return nullptr; }
+};
+
+// How the embedding's rows come back into the residual stream at chosen entries of the run order.
+class Reinjection : public Part {
+public:
+    using Part::Part;
+    // h [T, width] 32-bit, the stream, is replaced; x0 [T, width] 32-bit are the embedding's rows
+    virtual void forward(const Tensor& h, const Tensor& x0, Runtime& rt) = 0;
 };
 
 class PositionEncoding : public Part {
@@ -132,7 +143,7 @@ public:
 using PartFactory = std::function<std::unique_ptr<Part>(const PartSpec&)>;
 using BlockFactory = std::function<std::unique_ptr<Block>(const LayerSpec&)>;
 
-// role: norm, mixer, ffn, position, embedding, head, link
+// role: norm, mixer, ffn, position, embedding, head, link, reinjection
 void register_part(const std::string& role, const std::string& kind, PartFactory factory, bool replace = false);
 void register_block(const std::string& arrangement, BlockFactory factory, bool replace = false);
 std::unique_ptr<Part> build_part(const std::string& role, const PartSpec& spec);

@@ -13,10 +13,14 @@
 //          may itself be a part (an attention's "position")
 //   layer: {"mixer": part, "mixer_norm": part, "ffn": part, "ffn_norm": part,
 //           "arrangement": "pre_norm"}; an arrangement that joins a sub-layer to the residual
-//           stream by a part of its own names them as "mixer_link" and "ffn_link"
+//           stream by a part of its own names them as "mixer_link" and "ffn_link"; one that norms
+//           a sub-layer's output before the addition names those norms "mixer_post_norm" and
+//           "ffn_post_norm"
 //   model: {"architecture", "vocab_size", "hidden_size", "max_context", "streams" (residual
 //           streams per row, 1 if absent), "embedding": part,
-//           "layers": [layer], "order": [{"layer": i, "kv_from": j or null}],
+//           "layers": [layer], "order": [{"layer": i, "kv_from": j or null, "reinject": bool}],
+//           "reinjection": part (how the embedding's rows come back into the stream before the
+//           entries of the order that say "reinject"; absent: never),
 //           "final_norm": part, "head": part, "eos_token_ids": [..], "bos_token_id"}
 #pragma once
 #include <map>
@@ -79,6 +83,8 @@ struct LayerSpec {
     // how each sub-layer reads from and writes to the residual stream(s), for arrangements in
     // which that is a part with weights of its own (kind empty: the arrangement has none)
     PartSpec mixer_link, ffn_link;
+    // norms of the sub-layers' outputs, for arrangements that norm before and after (kind empty: none)
+    PartSpec mixer_post_norm, ffn_post_norm;
     std::string arrangement = "pre_norm";
 };
 
@@ -89,6 +95,9 @@ struct LayerSpec {
 struct RunStep {
     int layer = 0;
     std::optional<int> kv_from;
+    // before this entry runs, the stream is replaced by the model's reinjection part's mixture of
+    // the stream and the embedding's rows
+    bool reinject = false;
 };
 
 struct ModelSpec {
@@ -96,6 +105,7 @@ struct ModelSpec {
     int vocab_size = 0, hidden_size = 0, max_context = 0;
     int streams = 1;             // residual streams a row keeps between layers
     PartSpec embedding;
+    PartSpec reinjection;        // kind empty: the model has none
     std::vector<LayerSpec> layers;
     std::vector<RunStep> order;
     PartSpec final_norm, head;
@@ -112,6 +122,8 @@ struct ModelSpec {
                 throw SpecError("run order entry " + std::to_string(i) + " names layer " +
                                 std::to_string(order[i].layer) + ", but the model has " +
                                 std::to_string(layers.size()) + " layers");
+            if (order[i].reinject && reinjection.kind.empty())
+                throw SpecError("run order entry " + std::to_string(i) + " asks for the embedding's rows again, but the model names no \"reinjection\" part");
             if (order[i].kv_from && (*order[i].kv_from < 0 || *order[i].kv_from >= static_cast<int>(i)))
                 throw SpecError("run order entry " + std::to_string(i) + " reads the cache of entry " +
                                 std::to_string(*order[i].kv_from) + ", which does not run before it");
@@ -126,12 +138,19 @@ struct ModelSpec {
                           .set("arrangement", l.arrangement);
             if (!l.mixer_link.kind.empty()) lj.set("mixer_link", l.mixer_link.to_json());
             if (!l.ffn_link.kind.empty()) lj.set("ffn_link", l.ffn_link.to_json());
+            if (!l.mixer_post_norm.kind.empty()) lj.set("mixer_post_norm", l.mixer_post_norm.to_json());
+            if (!l.ffn_post_norm.kind.empty()) lj.set("ffn_post_norm", l.ffn_post_norm.to_json());
             ls.push(lj);
         }
         Json ord = Json::array();
-        for (const auto& s : order)
-            ord.push(Json::object().set("layer", s.layer).set("kv_from", s.kv_from ? Json(*s.kv_from) : Json()));
-        return Json::object().set("architecture", architecture).set("vocab_size", vocab_size)
+        for (const auto& s : order) {
+            Json e = Json::object().set("layer", s.layer).set("kv_from", s.kv_from ? Json(*s.kv_from) : Json());
+            if (s.reinject) e.set("reinject", true);
+            ord.push(e);
+        }
+        Json out = Json::object();
+        if (!reinjection.kind.empty()) out.set("reinjection", reinjection.to_json());
+        return out.set("architecture", architecture).set("vocab_size", vocab_size)
             .set("hidden_size", hidden_size).set("max_context", max_context).set("streams", streams)
             .set("embedding", embedding.to_json()).set("layers", ls).set("order", ord)
             .set("final_norm", final_norm.to_json()).set("head", head.to_json())
@@ -148,6 +167,7 @@ struct ModelSpec {
         m.max_context = static_cast<int>(j.get_int("max_context", 0));
         m.streams = static_cast<int>(j.get_int("streams", 1));
         m.embedding = PartSpec::from_json(j["embedding"], "embedding");
+        if (!j["reinjection"].is_null()) m.reinjection = PartSpec::from_json(j["reinjection"], "reinjection");
         if (!j["layers"].is_array()) throw SpecError("\"layers\" must be an array");
         int n = 0;
         for (const Json& l : j["layers"].items()) {
@@ -159,6 +179,8 @@ struct ModelSpec {
             ls.ffn_norm = PartSpec::from_json(l["ffn_norm"], where + ".ffn_norm");
             if (!l["mixer_link"].is_null()) ls.mixer_link = PartSpec::from_json(l["mixer_link"], where + ".mixer_link");
             if (!l["ffn_link"].is_null()) ls.ffn_link = PartSpec::from_json(l["ffn_link"], where + ".ffn_link");
+            if (!l["mixer_post_norm"].is_null()) ls.mixer_post_norm = PartSpec::from_json(l["mixer_post_norm"], where + ".mixer_post_norm");
+            if (!l["ffn_post_norm"].is_null()) ls.ffn_post_norm = PartSpec::from_json(l["ffn_post_norm"], where + ".ffn_post_norm");
             ls.arrangement = l.get_string("arrangement", "pre_norm");
             m.layers.push_back(std::move(ls));
         }
@@ -167,6 +189,7 @@ struct ModelSpec {
                 RunStep step;
                 step.layer = static_cast<int>(s.is_object() ? s.get_int("layer", -1) : s.as_int());
                 if (s.is_object() && !s["kv_from"].is_null()) step.kv_from = static_cast<int>(s["kv_from"].as_int());
+                if (s.is_object()) step.reinject = s.get_bool("reinject", false);
                 m.order.push_back(step);
             }
         } else {
