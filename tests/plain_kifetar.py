@@ -12,11 +12,20 @@ convolutions); a range of layers that runs several times, before every run of wh
 stream is mixed with the embedding's rows again; final layer norm; logits from the
 embedding table.
 """
+import json
 import math
+import os
 
 import torch
+from safetensors.torch import load_file
 
 F64 = torch.float64
+
+
+def load_model_folder(folder):
+    with open(os.path.join(folder, "config.json")) as fh:
+        cfg = json.load(fh)
+    return cfg, {k: v.to(F64) for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
 
 
 def layer_norm(x, w, b, eps):
@@ -167,3 +176,10 @@ def forward(config, tensors, tokens, return_layers=False):
         after.append(x.clone())
     logits = layer_norm(x, t["final.norm"], t["final.norm.b"], eps) @ t["embed"].T
     return (logits, torch.stack(after)) if return_layers else logits
+
+
+def greedy(config, tensors, prompt, n_new):
+    tokens = list(prompt)
+    for _ in range(n_new):
+        tokens.append(int(forward(config, tensors, tokens)[-1].argmax()))
+    return tokens[len(prompt):]
