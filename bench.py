@@ -138,27 +138,49 @@ def regipel_shape(width, layers, heads, dim, rot, vdim, rank, experts, top, ff, 
             "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": mlp} for _ in range(layers)]}
 
 
+# Kifetar likewise, beside LFM2 with a short convolution where Kifetar has a delta-rule layer and
+# attention where it has attention (same width, heads, feed-forward and vocabulary).
+def kifetar_shape(width, pattern, heads, kv_heads, dim, window, d_heads, d_kv_heads, d_dim, d_vdim, ff, vocab=65536):
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": window},
+                 "rot": {"base": 500000.0, "dims": dim // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    delta = {"heads": d_heads, "kv_heads": d_kv_heads, "dim": d_dim, "vdim": d_vdim, "conv": 4}
+    mlp = {"kind": "dense", "ff": ff}
+    return {"architecture": "Kifetar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "max_context": 8192,
+            "layers": [{"type": "attention", "mixer": attention, "mlp": mlp} if kind == "a" else
+                       {"type": "delta", "mixer": delta, "mlp": mlp} for kind in pattern]}
+
+
+KIFETAR_PATTERN = "daadaada"
+KIFETAR_ATTENTION = {i for i, kind in enumerate(KIFETAR_PATTERN) if kind == "a"}
+KIFETAR_SHAPES = {
+    "1k": (kifetar_shape(1024, KIFETAR_PATTERN, 16, 8, 64, 1024, 16, 8, 64, 64, 2048),
+           lfm2_shape(1024, 16, 8, 2048, KIFETAR_ATTENTION, 8, 8192)),
+    "2k": (kifetar_shape(2048, KIFETAR_PATTERN, 32, 8, 64, 1024, 16, 8, 128, 128, 4096),
+           lfm2_shape(2048, 32, 8, 4096, KIFETAR_ATTENTION, 8, 8192)),
+}
+
 DESIGN_SHAPES = {
     "1k": (regipel_shape(1024, 8, 16, 64, 32, 64, 256, 16, 2, 1024), lfm2_shape(1024, 16, 8, 2048, set(range(8)), 8, 8192)),
     "2k": (regipel_shape(2048, 8, 16, 128, 64, 128, 512, 32, 4, 1024), lfm2_shape(2048, 32, 8, 4096, set(range(8)), 8, 8192)),
 }
 
 
-def design(shapes, steps: int, warmup: int, batch: int, layers: int = 0, profile_only: str = "") -> int:
+def design(shapes, steps: int, warmup: int, batch: int, layers: int = 0, profile_only: str = "", which: str = "regipel") -> int:
     """Prefill of 2,048 tokens and decode at `batch` requests of 2,048 tokens, for every shape and
-    both models.  Prints one JSON line."""
+    both models (the design `which` and the LFM2 shape beside it).  Prints one JSON line."""
     import torch
     from celeg_amd.engine import Engine
     from celeg_amd.engine.benchmark import DecodeBench, measure_prefill
     from celeg_amd.weights import write_random_model
     out = {}
     for shape in shapes:
-        for label, cfg in zip(("regipel", "lfm2_attention"), DESIGN_SHAPES[shape]):
+        table, beside = (KIFETAR_SHAPES, "lfm2_hybrid") if which == "kifetar" else (DESIGN_SHAPES, "lfm2_attention")
+        for label, cfg in zip((which, beside), table[shape]):
             if profile_only and label != profile_only:
                 continue
             cfg = json.loads(json.dumps(cfg))
             if layers:
-                if label == "regipel":
+                if label == which:
                     cfg["layers"] = cfg["layers"][:layers]
                 else:
                     cfg.update(num_hidden_layers=layers, layer_types=cfg["layer_types"][:layers])
@@ -182,9 +204,10 @@ def design(shapes, steps: int, warmup: int, batch: int, layers: int = 0, profile
                 "weights": lm.native.info["weights"], "kv_bytes_per_token": lm.native.info["kv_bytes_per_token"],
                 "layers": len(lm.native.info["spec"]["order"])}
             engine.close()
-    print(json.dumps({"metric": "Regipel beside LFM2 attention layers at equal size: prefill tok/s @ 2048 tokens, "
+    title = "Kifetar beside LFM2 convolution and attention layers" if which == "kifetar" else "Regipel beside LFM2 attention layers"
+    print(json.dumps({"metric": title + " at equal size: prefill tok/s @ 2048 tokens, "
                                 f"decode tok/s @ batch {batch}, context 2048 (bf16, random weights)",
-                      "phase": "design", "batch": batch, "steps": steps, "warmup": warmup, "dtype": "bf16",
+                      "phase": "design", "design": which, "batch": batch, "steps": steps, "warmup": warmup, "dtype": "bf16",
                       "data": "synthetic", "shapes": out}))
     return 0
 
@@ -211,7 +234,9 @@ def main() -> int:
                          "(default 2048, the headline's); with --phase prefill: tokens of the same "
                          "prompt that the cache holds before the measured portion of 2,048 (default 0)")
     ap.add_argument("--design-shape", default="1k,2k", help="with --phase design: which sizes (1k, 2k)")
-    ap.add_argument("--design-model", default="", choices=["", "regipel", "lfm2_attention"],
+    ap.add_argument("--design", default="regipel", choices=["regipel", "kifetar"],
+                    help="with --phase design: which design is measured beside its closest LFM2 shape")
+    ap.add_argument("--design-model", default="", choices=["", "regipel", "lfm2_attention", "kifetar", "lfm2_hybrid"],
                     help="with --phase design: only this model (for profiling)")
     ap.add_argument("--phase", choices=["all", "prefill", "decode", "serve", "design"], default="all",
                     help="for profiling: run only the prefill measurement, or only the batch-8 "
@@ -231,7 +256,7 @@ def main() -> int:
 
     if args.phase == "design":
         return design(args.design_shape.split(","), min(args.steps, 64), min(args.warmup, 8), args.batch, args.layers,
-                      args.design_model)
+                      args.design_model, args.design)
     if args.phase == "serve":
         return serve(args.shape, args.prefill_chunk, args.token_budget, args.portion_granule, args.gemm_backend)
 

@@ -151,6 +151,99 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_kernel(
         for (int d = 0; d < D; ++d) mine[static_cast<size_t>(d) * V + j] = S[d * CELEG_WAVE + lane];
 }
 
+// The same recurrence with S in registers, for dim = 16 * DL: DL neighbouring lanes share a column
+// of S, each holding 16 of its values, so a wavefront owns 64 / DL columns and the sums over dim
+// meet by DL - 1 exchanges between neighbours.  The rows of a request are taken in blocks of TB
+// tokens: a block's q, k, write strengths and decays are staged in LDS (asked for from memory while
+// the block before is computed), its values sit in registers.  With u = beta (v - a (S^T k)) the
+// new column is a S + k u, read out with q in the same pass.
+template <int DL>
+__global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
+    const float* __restrict__ qk, const float* __restrict__ v, const float* __restrict__ beta_decay, float* __restrict__ state,
+    size_t state_stride, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot, float* __restrict__ out, int G, int H,
+    int V) {
+    constexpr int D = 16 * DL, CPW = CELEG_WAVE / DL, TB = D <= 64 ? 16 : 8, ROW = 2 * D, PER_LANE = TB * ROW / CELEG_WAVE;
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) float qk_s[TB * ROW];
+    __shared__ float bd_s[TB * 2];
+    const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int sub = lane % DL, j = blockIdx.z * CPW + lane / DL;
+    const bool live = j < V;
+    const int jj = live ? j : V - 1;          // idle lanes repeat the last column and store nothing
+    const int g = h / (H / G);
+    const int row0 = cu_seqlens[s], n = cu_seqlens[s + 1] - row0;
+    if (n <= 0) return;
+    float* mine = state + static_cast<size_t>(seq_slot[s]) * state_stride + static_cast<size_t>(h) * D * V;
+    float S[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) S[i] = mine[static_cast<size_t>(sub * 16 + i) * V + jj];
+    const size_t ldqk = static_cast<size_t>(2) * G * D;
+    float pre[PER_LANE], pre_v[TB], pre_bd = 0.f;
+    auto fetch = [&](int block) __attribute__((always_inline)) {
+        const int t0 = block * TB;
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) {
+            const int e = lane + CELEG_WAVE * i, tt = e / ROW, x = e % ROW;
+            const int t = min(t0 + tt, n - 1);
+            pre[i] = qk[static_cast<size_t>(row0 + t) * ldqk + (x < D ? g * D + x : (G + g) * D + x - D)];
+        }
+#pragma unroll
+        for (int tt = 0; tt < TB; ++tt) pre_v[tt] = v[static_cast<size_t>(row0 + min(t0 + tt, n - 1)) * H * V + static_cast<size_t>(h) * V + jj];
+        if (lane < 2 * TB) pre_bd = beta_decay[static_cast<size_t>(row0 + min(t0 + lane / 2, n - 1)) * 2 * H + (lane & 1) * H + h];
+    };
+    fetch(0);
+    const int n_blocks = (n + TB - 1) / TB;
+    for (int block = 0; block < n_blocks; ++block) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) qk_s[lane + CELEG_WAVE * i] = pre[i];
+        if (lane < 2 * TB) bd_s[lane] = pre_bd;
+        float vals[TB];
+#pragma unroll
+        for (int tt = 0; tt < TB; ++tt) vals[tt] = pre_v[tt];
+        __syncthreads();
+        if (block + 1 < n_blocks) fetch(block + 1);
+        const int count = min(TB, n - block * TB);
+#pragma unroll
+        for (int tt = 0; tt < TB; ++tt) {
+            if (tt >= count) break;
+            const float* qrow = qk_s + tt * ROW + sub * 16;
+            f4 q4[4], k4[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                q4[c] = *reinterpret_cast<const f4*>(qrow + 4 * c);
+                k4[c] = *reinterpret_cast<const f4*>(qrow + D + 4 * c);
+            }
+            const float beta = bd_s[2 * tt], decay = bd_s[2 * tt + 1];
+            float part[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) part[e] = fmaf(k4[c][e], S[4 * c + e], part[e]);
+            float kv = (part[0] + part[1]) + (part[2] + part[3]);
+#pragma unroll
+            for (int off = 1; off < DL; off <<= 1) kv += __shfl_xor(kv, off, CELEG_WAVE);
+            const float u = beta * (vals[tt] - decay * kv);
+            float opart[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float sd = fmaf(k4[c][e], u, decay * S[4 * c + e]);
+                    S[4 * c + e] = sd;
+                    opart[e] = fmaf(q4[c][e], sd, opart[e]);
+                }
+            float o = (opart[0] + opart[1]) + (opart[2] + opart[3]);
+#pragma unroll
+            for (int off = 1; off < DL; off <<= 1) o += __shfl_xor(o, off, CELEG_WAVE);
+            if (live && sub == 0) out[static_cast<size_t>(row0 + block * TB + tt) * H * V + static_cast<size_t>(h) * V + j] = o;
+        }
+    }
+    if (live)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mine[static_cast<size_t>(sub * 16 + i) * V + j] = S[i];
+}
+
 // one wavefront per (row, head): out = o / sqrt(mean(o^2) + eps) * w * silu(gate)
 template <typename T>
 __global__ __launch_bounds__(CELEG_WAVE) void delta_gated_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
@@ -204,8 +297,23 @@ extern "C" int celeg_delta_conv_state(const void* proj, int ld, int dtype, float
 
 extern "C" int celeg_delta_scan(const float* qk, const float* v, const float* beta_decay, float* state, size_t state_stride,
                                 const int* cu_seqlens, const int* seq_slot, float* out, int n_seqs, int G, int H, int D, int V,
-                                hipStream_t stream) {
+                                int general, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
+    if (H % G) return static_cast<int>(hipErrorInvalidValue);
+    if (!general && (D == 16 || D == 32 || D == 64 || D == 128 || D == 256)) {
+        const int DL = D / 16, cpw = CELEG_WAVE / DL;
+        dim3 grid(n_seqs, H, (V + cpw - 1) / cpw), block(CELEG_WAVE);
+#define CELEG_DELTA_REG(DL_)                                                                                                  \
+    hipLaunchKernelGGL(delta_scan_reg_kernel<DL_>, grid, block, 0, stream, qk, v, beta_decay, state, state_stride, cu_seqlens, \
+                       seq_slot, out, G, H, V)
+        if (DL == 1) CELEG_DELTA_REG(1);
+        else if (DL == 2) CELEG_DELTA_REG(2);
+        else if (DL == 4) CELEG_DELTA_REG(4);
+        else if (DL == 8) CELEG_DELTA_REG(8);
+        else CELEG_DELTA_REG(16);
+#undef CELEG_DELTA_REG
+        return CELEG_LAUNCH_RESULT();
+    }
     const size_t lds = (static_cast<size_t>(D) * CELEG_WAVE + 2 * static_cast<size_t>(D)) * sizeof(float);
     if (lds > 64 * 1024 || H % G) return static_cast<int>(hipErrorInvalidValue);
     dim3 grid(n_seqs, H, (V + CELEG_WAVE - 1) / CELEG_WAVE), block(CELEG_WAVE);

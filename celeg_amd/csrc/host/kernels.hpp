@@ -152,6 +152,12 @@ int celeg_sigmoid_attention(const void* q, int ldq, const void* k_pool, const vo
                             const float* bias, const void* gate, int ldg, void* out, int ldo, int n_tokens, int q_heads,
                             int kv_heads, int head_dim, int page_tokens, int n_layers, int layer, float scale, int window,
                             hipStream_t stream);
+int celeg_sigmoid_attention_fast_ok(int head_dim);
+int celeg_sigmoid_attention_fast(const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
+                                 int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start, int n_seqs,
+                                 int max_tiles, const float* temp, const float* bias, const void* gate, int ldg, void* out,
+                                 int ldo, int q_heads, int kv_heads, int head_dim, int page_tokens, int n_layers, int layer,
+                                 float scale, int window, hipStream_t stream);
 // delta_rule.hip
 int celeg_delta_prepare(const void* proj, int ld, int dtype, int col_b, int col_a, const float* conv_w, const float* a_log,
                         const float* dt_bias, const float* conv_state, size_t state_stride, const int* positions,
@@ -161,7 +167,7 @@ int celeg_delta_conv_state(const void* proj, int ld, int dtype, float* conv_stat
                            const int* seq_slot, int n_seqs, int n_channels, int taps, hipStream_t stream);
 int celeg_delta_scan(const float* qk, const float* v, const float* beta_decay, float* state, size_t state_stride,
                      const int* cu_seqlens, const int* seq_slot, float* out, int n_seqs, int G, int H, int D, int V,
-                     hipStream_t stream);
+                     int general, hipStream_t stream);
 int celeg_delta_gated_norm(const float* o, const float* w, const void* gate, int ldg, int dtype, float eps, void* out,
                            int n_tokens, int H, int V, hipStream_t stream);
 }

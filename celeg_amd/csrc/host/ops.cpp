@@ -762,6 +762,20 @@ void Ops::sigmoid_attention(const Tensor& q, const Tensor& out, int heads, int k
         ldg = rows_of(*gate, "gate");
     }
     took(Path::AttentionSigmoid);
+    const int ldq = rows_of(q, "q");
+    if (q.dtype == DType::BF16 && use_sigmoid_mfma && !attention_general && celeg_sigmoid_attention_fast_ok(head_dim) &&
+        kv.page_tokens >= 8 && (kv.page_tokens & (kv.page_tokens - 1)) == 0 && ldq % 8 == 0 && head_dim % 8 == 0 &&
+        (reinterpret_cast<uintptr_t>(q.data) & 15) == 0) {
+        // tiles of 16 rows: at most one partly filled tile per request
+        const int max_tiles = static_cast<int>(T) / 16 + batch.n_seqs;
+        took(batch.decode_only ? Path::AttentionSigmoidDecode : Path::AttentionSigmoidRows);
+        kernel_check(celeg_sigmoid_attention_fast(q.data, ldq, kv.k, kv.v, kv.table, kv.table_stride, batch.cu_seqlens, batch.seq_slot,
+                                                  batch.seq_start, batch.n_seqs, max_tiles, temp ? temp->as<float>() : nullptr,
+                                                  bias ? bias->as<float>() : nullptr, gate ? gate->data : nullptr, ldg, out.data,
+                                                  static_cast<int>(qw), heads, kv_heads, head_dim, kv.page_tokens, kv.n_layers, kv.layer,
+                                                  scale, window, stream), "sigmoid attention (bfloat16, matrix cores)");
+        return;
+    }
     kernel_check(celeg_sigmoid_attention(q.data, rows_of(q, "q"), kv.k, kv.v, dt(q, "q"), kv.table, kv.table_stride, batch.token_slot,
                                          batch.positions, temp ? temp->as<float>() : nullptr, bias ? bias->as<float>() : nullptr,
                                          gate ? gate->data : nullptr, ldg, out.data, static_cast<int>(qw), static_cast<int>(T), heads,
@@ -816,10 +830,10 @@ void Ops::delta_scan(const Tensor& qk, const Tensor& v, const Tensor& beta_decay
              beta_decay.numel() == T * 2 * s.heads, "delta_scan: rows do not fit");
     need(state.ndim >= 2 && state.numel() / state.shape[0] == per_slot && state.stride[state.ndim - 1] == 1,
          "delta_scan: state must be [slots, heads, dim, vdim]");
-    need((static_cast<long long>(s.dim) * 64 + 2 * s.dim) * 4 <= 64 * 1024, "delta_scan: dim " + std::to_string(s.dim) + " exceeds 248");
+    need(s.dim <= 256 && (s.dim <= 248 || s.dim == 256), "delta_scan: dim " + std::to_string(s.dim) + " exceeds 256");
     kernel_check(celeg_delta_scan(qk.as<float>(), v.as<float>(), beta_decay.as<float>(), state.as<float>(),
                                   static_cast<size_t>(state.stride[0]), batch.cu_seqlens, batch.seq_slot, out.as<float>(), batch.n_seqs,
-                                  s.kv_heads, s.heads, s.dim, s.vdim, stream), "delta_scan");
+                                  s.kv_heads, s.heads, s.dim, s.vdim, delta_general ? 1 : 0, stream), "delta_scan");
 }
 
 void Ops::delta_gated_norm(const Tensor& o, const Tensor& weight, const Tensor& gate, float eps, const Tensor& out, int heads, int vdim) {

@@ -123,6 +123,8 @@ public:
     int decode_split_rounds(long long groups, int rounds) const;
     bool decode_whole(long long groups, int rounds) const;
     bool attention_general = false;      // always the general attention kernel
+    bool delta_general = false;          // the delta rule's recurrence always by the kernel for any dim
+    bool use_sigmoid_mfma = true;        // bfloat16 attention with sigmoid weights on the matrix cores
     bool use_router_kernel = true;       // the router's product inside the routing kernel
     bool use_moe_mfma = true;            // bfloat16 products of routed experts and per-head matrices on the matrix cores
     bool use_latent_mfma = true;         // bfloat16 attention over a latent cache on the matrix cores

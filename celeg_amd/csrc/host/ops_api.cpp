@@ -158,6 +158,8 @@ void set_knobs(Ops& ops, const Json& knobs) {
         else if (name == "decode_parts_some") ops.decode_part_thresholds[1] = static_cast<int>(v);
         else if (name == "attention_general") ops.attention_general = v != 0;
         else if (name == "use_rope_table") ops.use_rope_table = v != 0;
+        else if (name == "delta_general") ops.delta_general = v != 0;
+        else if (name == "use_sigmoid_mfma") ops.use_sigmoid_mfma = v != 0;
         else if (name == "use_argmax_parts") ops.use_argmax_parts = v != 0;
         else if (name == "use_head_argmax") ops.use_head_argmax = v != 0;
         else if (name == "decode_parts_fill") ops.decode_parts_fill = v != 0;

@@ -82,6 +82,144 @@ __global__ __launch_bounds__(CELEG_WAVE) void sigmoid_attention_kernel(
     }
 }
 
+// ---------------------------------------------------------------- bfloat16 on the matrix cores
+// One wavefront per (16 rows of one request's step, query head); a workgroup holds four such
+// wavefronts that share nothing.  The wavefront walks the keys its rows can see, 64 at a time,
+// from the first key of its first row's window (rounded down to 8, which stays inside that key's
+// page) to its last row's position: the block's keys [64][D] and values [D][64] (as the pages hold
+// them) go through the wavefront's own part of LDS.  Scores are computed transposed (keys as the
+// first operand), so a lane ends up with four neighbouring keys of one row in each of the block's
+// four tiles; two tiles' weights, rounded to bfloat16, are then a lane's second operand of the
+// product with the values as they are, the eight keys dealt to the instruction in the order the
+// lane holds them, and the values' operand reads the same eight keys.  Sums are 32-bit; the
+// order of a row's additions depends on the row's place in its 16 rows and its position only.
+typedef __bf16 sa_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 sa_bf16x4 __attribute__((ext_vector_type(4)));
+typedef float sa_f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int sa_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int sa_u32x2 __attribute__((ext_vector_type(2)));
+
+#define SA_WAVES 4
+#define SA_KEYS 64
+
+template <int D>
+__global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_kernel(
+    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
+    const int* __restrict__ table, int table_stride, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_start, int n_seqs, const float* __restrict__ temp, const float* __restrict__ bias,
+    const bf16* __restrict__ gate, int ldg, bf16* __restrict__ out, int ldo, int q_heads, int kv_heads, int page_tokens,
+    int n_layers, int layer, float scale, int window) {
+    constexpr int KROW = D + 8, VROW = SA_KEYS + 8;      // padded rows: neighbouring rows start in different banks
+    constexpr int KS = D / 32, DT = D / 16;
+    extern __shared__ __attribute__((aligned(16))) unsigned char sa_lds[];
+    const int wave = threadIdx.x / CELEG_WAVE, lane = threadIdx.x % CELEG_WAVE;
+    __bf16* ks = reinterpret_cast<__bf16*>(sa_lds) + static_cast<size_t>(wave) * (SA_KEYS * KROW + D * VROW);
+    __bf16* vs = ks + SA_KEYS * KROW;
+    // which 16 rows: tiles of all requests of the step, one after the other
+    int tile = blockIdx.x * SA_WAVES + wave, s = 0, row0 = 0, n = 0;
+    for (; s < n_seqs; ++s) {
+        row0 = cu_seqlens[s];
+        n = cu_seqlens[s + 1] - row0;
+        const int tiles = (n + 15) / 16;
+        if (tile < tiles) break;
+        tile -= tiles;
+    }
+    if (s >= n_seqs) return;
+    const int h = blockIdx.y, kvh = h / (q_heads / kv_heads);
+    const int r = lane & 15, quad = lane >> 4;
+    const int first_row = tile * 16, rows_here = min(16, n - first_row);
+    const int pos0 = seq_start[s] + first_row, pos_last = pos0 + rows_here - 1;
+    const int my_row = first_row + min(r, rows_here - 1);      // rows past the end repeat the last one (not stored)
+    const int my_pos = seq_start[s] + my_row;
+    const int* pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
+    const float tau = scale * (temp ? temp[h] : 1.0f), beta = bias ? bias[h] : 0.0f;
+    // this lane's operand of q: row r, values 32 st + 8 quad .. + 8
+    sa_bf16x8 qreg[KS];
+    const bf16* qrow = q + static_cast<size_t>(row0 + my_row) * ldq + static_cast<size_t>(h) * D;
+#pragma unroll
+    for (int st = 0; st < KS; ++st) qreg[st] = __builtin_bit_cast(sa_bf16x8, *reinterpret_cast<const sa_u32x4*>(qrow + 32 * st + 8 * quad));
+    sa_f32x4 oacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
+    const int key_first = window > 0 ? max(0, pos0 - window + 1) : 0;
+    const size_t head_stride = static_cast<size_t>(page_tokens) * D;
+    for (int kb = key_first & ~7; kb <= pos_last; kb += SA_KEYS) {
+        // stage: keys kb .. kb + 63 (those past pos_last: the last one again), values with zeros past pos_last
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (int c = lane; c < SA_KEYS * (D / 8); c += CELEG_WAVE) {
+            const int key_in = c / (D / 8), part = c % (D / 8);
+            const int key = min(kb + key_in, pos_last);
+            const bf16* src = k_pool + ((static_cast<size_t>(pages[key / page_tokens]) * n_layers + layer) * kv_heads + kvh) * head_stride +
+                              static_cast<size_t>(key % page_tokens) * D + 8 * part;
+            *reinterpret_cast<sa_u32x4*>(ks + key_in * KROW + 8 * part) = *reinterpret_cast<const sa_u32x4*>(src);
+        }
+        for (int c = lane; c < D * (SA_KEYS / 8); c += CELEG_WAVE) {
+            const int d = c / (SA_KEYS / 8), part = c % (SA_KEYS / 8);
+            const int key = kb + 8 * part;         // eight keys that lie side by side in one page
+            sa_u32x4 val = {0u, 0u, 0u, 0u};
+            if (key <= pos_last) {
+                const bf16* src = v_pool + ((static_cast<size_t>(pages[key / page_tokens]) * n_layers + layer) * kv_heads + kvh) * head_stride +
+                                  static_cast<size_t>(d) * page_tokens + key % page_tokens;
+                val = *reinterpret_cast<const sa_u32x4*>(src);
+                const int live = pos_last - key + 1;       // keys of this piece that exist
+                if (live < 8) {
+                    if (live <= 6) val[3] = 0u; else val[3] &= 0x0000ffffu;
+                    if (live <= 4) val[2] = 0u; else if (live == 5) val[2] &= 0x0000ffffu;
+                    if (live <= 2) val[1] = 0u; else if (live == 3) val[1] &= 0x0000ffffu;
+                    if (live == 1) val[0] &= 0x0000ffffu;
+                }
+            }
+            *reinterpret_cast<sa_u32x4*>(vs + d * VROW + 8 * part) = val;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // scores, transposed: tile kt holds keys kb + 16 kt + 4 quad + i of row r
+        sa_f32x4 sacc[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            sacc[kt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int st = 0; st < KS; ++st) {
+                const sa_bf16x8 kf = __builtin_bit_cast(sa_bf16x8, *reinterpret_cast<const sa_u32x4*>(ks + (16 * kt + r) * KROW + 32 * st + 8 * quad));
+                sacc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qreg[st], sacc[kt], 0, 0, 0);
+            }
+        }
+        // weights: sigmoid inside the row's window, nothing outside
+        sa_bf16x4 w[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kb + 16 * kt + 4 * quad + i;
+                const bool seen = key <= my_pos && (window <= 0 || key > my_pos - window);
+                w[kt][i] = static_cast<__bf16>(seen ? sa_sigmoid(sacc[kt][i] * tau + beta) : 0.0f);
+            }
+        // output, transposed: tile dt holds values 16 dt + 4 quad + i of row r
+#pragma unroll
+        for (int pair = 0; pair < 2; ++pair) {
+            const sa_bf16x8 pw = __builtin_shufflevector(w[2 * pair], w[2 * pair + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const __bf16* vrow = vs + (16 * dt + r) * VROW + 32 * pair + 4 * quad;
+                const sa_u32x2 lo = *reinterpret_cast<const sa_u32x2*>(vrow), hi = *reinterpret_cast<const sa_u32x2*>(vrow + 16);
+                const sa_bf16x8 vf = __builtin_bit_cast(sa_bf16x8, sa_u32x4{lo[0], lo[1], hi[0], hi[1]});
+                oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pw, oacc[dt], 0, 0, 0);
+            }
+        }
+    }
+    if (r >= rows_here) return;
+    const float g = gate ? sa_sigmoid(to_float(gate[static_cast<size_t>(row0 + my_row) * ldg + h])) : 1.0f;
+    bf16* orow = out + static_cast<size_t>(row0 + my_row) * ldo + static_cast<size_t>(h) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const sa_bf16x4 o4 = {static_cast<__bf16>(oacc[dt][0] * g), static_cast<__bf16>(oacc[dt][1] * g),
+                              static_cast<__bf16>(oacc[dt][2] * g), static_cast<__bf16>(oacc[dt][3] * g)};
+        *reinterpret_cast<sa_bf16x4*>(orow + 16 * dt + 4 * quad) = o4;
+    }
+}
+
 }  // namespace
 
 extern "C" int celeg_sigmoid_attention(const void* q, int ldq, const void* k_pool, const void* v_pool, int dtype,
@@ -103,5 +241,33 @@ extern "C" int celeg_sigmoid_attention(const void* q, int ldq, const void* k_poo
                            static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table, table_stride, token_slot,
                            positions, temp, bias, static_cast<const bf16*>(gate), ldg, static_cast<bf16*>(out), ldo, q_heads,
                            kv_heads, head_dim, page_tokens, n_layers, layer, scale, window);
+    return CELEG_LAUNCH_RESULT();
+}
+
+// head sizes the matrix-core kernel takes
+extern "C" int celeg_sigmoid_attention_fast_ok(int head_dim) { return head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128; }
+
+// bfloat16 on the matrix cores; max_tiles: an upper bound on the step's tiles of 16 rows
+// (sum over requests of ceil(rows / 16)); pages of a power of two of at least 8 tokens
+extern "C" int celeg_sigmoid_attention_fast(const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
+                                            int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start,
+                                            int n_seqs, int max_tiles, const float* temp, const float* bias, const void* gate,
+                                            int ldg, void* out, int ldo, int q_heads, int kv_heads, int head_dim, int page_tokens,
+                                            int n_layers, int layer, float scale, int window, hipStream_t stream) {
+    if (max_tiles <= 0 || n_seqs <= 0) return 0;
+    if (!celeg_sigmoid_attention_fast_ok(head_dim) || q_heads % kv_heads || page_tokens % 8 || ldq % 8 || ldo % 4)
+        return static_cast<int>(hipErrorInvalidValue);
+    dim3 grid((max_tiles + SA_WAVES - 1) / SA_WAVES, q_heads), block(SA_WAVES * CELEG_WAVE);
+    const size_t lds = static_cast<size_t>(SA_WAVES) * (SA_KEYS * (head_dim + 8) + head_dim * (SA_KEYS + 8)) * 2;
+#define CELEG_SA_FAST(D_)                                                                                                        \
+    hipLaunchKernelGGL(sigmoid_attention_mfma_kernel<D_>, grid, block, lds, stream, static_cast<const bf16*>(q), ldq,               \
+                       static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table, table_stride, cu_seqlens, seq_slot, \
+                       seq_start, n_seqs, temp, bias, static_cast<const bf16*>(gate), ldg, static_cast<bf16*>(out), ldo, q_heads,    \
+                       kv_heads, page_tokens, n_layers, layer, scale, window)
+    if (head_dim == 32) CELEG_SA_FAST(32);
+    else if (head_dim == 64) CELEG_SA_FAST(64);
+    else if (head_dim == 96) CELEG_SA_FAST(96);
+    else CELEG_SA_FAST(128);
+#undef CELEG_SA_FAST
     return CELEG_LAUNCH_RESULT();
 }

@@ -227,6 +227,45 @@ def test_window_edges_in_prompts_and_decoding(tmp_path, dtype):
             assert_close(got[rid], ref[rid], dtype, f"windows/{dtype}/{rid}")
 
 
+@pytest.mark.parametrize("dim", [32, 64, 96, 128])
+def test_matrix_core_attention_equals_the_general_kernel(tmp_path, dim):
+    """bfloat16: the kernel on the matrix cores against the kernel that scores key by key, on the
+    same pages, with sharp weights and windows that end before, at and behind the borders of pages
+    and of the blocks of 64 keys, in whole prompts, portions and single tokens.  The two differ in
+    the rounding of the weights to bfloat16 only, so they are held to a fifth of what rounding does
+    to a whole model."""
+    cfg = {"architecture": "Kifetar", "vocab": 150, "width": 64, "norm": {"eps": 1e-5},
+           "layers": [attention(4, 2, dim, window=w, rot=rot(dim // 2, 500.0), ff=None) for w in (1, 7, 64, 65, 100, None)]}
+    folder = write_model(tmp_path / "mfma", cfg, 31, torch.bfloat16, std=0.1, change=sharp(cfg, 2.0))
+    reqs = {"a": random_tokens(cfg["vocab"], 300, seed=9), "b": random_tokens(cfg["vocab"], 75, seed=10), "c": random_tokens(cfg["vocab"], 16, seed=11)}
+    for steps in (whole_schedule(reqs), tail_decode_schedule(reqs, tail=15), portions_schedule(reqs, sizes=(15, 2, 17, 1, 130, 3, 16, 64)),
+                  mixed_schedule(reqs, seed=2, decode_tail=5)):
+        got = {}
+        for fast in (1, 0):
+            lm, _ = load(folder, "bfloat16", steps)
+            lm.set_knob("use_sigmoid_mfma", fast)
+            got[fast] = EngineDriver(lm).run(steps)
+            assert (lm.paths()["attention_sigmoid_rows"] > 0) == bool(fast)
+        for rid in reqs:
+            a, b = got[1][rid].double(), got[0][rid].double()
+            rel = float((a - b).pow(2).mean().sqrt() / b.pow(2).mean().sqrt())
+            assert rel <= 1.5e-2, f"head size {dim}, {rid}: rel rms {rel:.3e}"
+
+
+def test_delta_rule_in_registers_equals_the_general_kernel(folders):
+    """32-bit: the recurrence with the state in registers against the kernel for any size, same schedule."""
+    folder = folders("K4", "float32")
+    reqs = requests_of("K4")
+    steps = mixed_schedule(reqs, seed=6)
+    got = {}
+    for general in (0, 1):
+        lm, _ = load(folder, "float32", steps)
+        lm.set_knob("delta_general", general)
+        got[general] = EngineDriver(lm).run(steps)
+    for rid in reqs:
+        assert_close_f32(got[0][rid], got[1][rid], rid)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_state_that_remembers_hundreds_of_tokens(tmp_path, dtype):
     """Decays close to one: what the first tokens wrote into the state still shows 300 tokens
@@ -366,7 +405,9 @@ def test_sigmoid_attention_alone(tmp_path, window, scaling):
     assert_close_f32(got, Wd["x"] + plain.sigmoid_window_attention(Wd["x"], m, Wd, "", 1e-4), "sigmoid attention alone")
 
 
-@pytest.mark.parametrize("H,G,D,V,taps", [(4, 2, 12, 20, 3), (3, 3, 8, 70, 1), (2, 1, 40, 8, 6)])
+# (dims of 16, 32, 64, 128 and 256 keep the state in registers, 1, 2, 4, 8 and 16 lanes a column; the others do not)
+@pytest.mark.parametrize("H,G,D,V,taps", [(4, 2, 12, 20, 3), (3, 3, 8, 70, 1), (2, 1, 40, 8, 6), (4, 2, 16, 100, 4), (2, 2, 32, 64, 2),
+                                          (3, 1, 64, 48, 4), (2, 1, 128, 24, 2), (1, 1, 256, 70, 3)])
 def test_gated_delta_rule_alone(tmp_path, H, G, D, V, taps):
     torch.manual_seed(2)
     T, W_ = 45, 32
