@@ -151,9 +151,24 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_kernel(
         for (int d = 0; d < D; ++d) mine[static_cast<size_t>(d) * V + j] = S[d * CELEG_WAVE + lane];
 }
 
+// The sum of v over every group of W neighbouring lanes (1 to 16), in all of them, by the vector
+// unit's cross-lane modifiers: lanes swapped in pairs and in pairs of pairs, then the halves of 8
+// and of 16 mirrored.  Both sides of every exchange add the same two numbers, so the lanes agree.
+template <int W>
+__device__ __forceinline__ float lanes_sum(float v) {
+    auto across = [](float x, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, false));
+    };
+    if (W >= 2) v += across(v, std::integral_constant<int, 0xB1>{});
+    if (W >= 4) v += across(v, std::integral_constant<int, 0x4E>{});
+    if (W >= 8) v += across(v, std::integral_constant<int, 0x141>{});
+    if (W >= 16) v += across(v, std::integral_constant<int, 0x140>{});
+    return v;
+}
+
 // The same recurrence with S in registers, for dim = 16 * DL: DL neighbouring lanes share a column
 // of S, each holding 16 of its values, so a wavefront owns 64 / DL columns and the sums over dim
-// meet by DL - 1 exchanges between neighbours.  The rows of a request are taken in blocks of TB
+// meet by log2(DL) exchanges between neighbours.  The rows of a request are taken in blocks of TB
 // tokens: a block's q, k, write strengths and decays are staged in LDS (asked for from memory while
 // the block before is computed), its values sit in registers.  With u = beta (v - a (S^T k)) the
 // new column is a S + k u, read out with q in the same pass.
@@ -220,9 +235,7 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
             for (int c = 0; c < 4; ++c)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) part[e] = fmaf(k4[c][e], S[4 * c + e], part[e]);
-            float kv = (part[0] + part[1]) + (part[2] + part[3]);
-#pragma unroll
-            for (int off = 1; off < DL; off <<= 1) kv += __shfl_xor(kv, off, CELEG_WAVE);
+            const float kv = lanes_sum<DL>((part[0] + part[1]) + (part[2] + part[3]));
             const float u = beta * (vals[tt] - decay * kv);
             float opart[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -233,9 +246,7 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
                     S[4 * c + e] = sd;
                     opart[e] = fmaf(q4[c][e], sd, opart[e]);
                 }
-            float o = (opart[0] + opart[1]) + (opart[2] + opart[3]);
-#pragma unroll
-            for (int off = 1; off < DL; off <<= 1) o += __shfl_xor(o, off, CELEG_WAVE);
+            const float o = lanes_sum<DL>((opart[0] + opart[1]) + (opart[2] + opart[3]));
             if (live && sub == 0) out[static_cast<size_t>(row0 + block * TB + tt) * H * V + static_cast<size_t>(h) * V + j] = o;
         }
     }

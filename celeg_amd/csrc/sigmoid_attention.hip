@@ -83,11 +83,13 @@ __global__ __launch_bounds__(CELEG_WAVE) void sigmoid_attention_kernel(
 }
 
 // ---------------------------------------------------------------- bfloat16 on the matrix cores
-// One wavefront per (16 rows of one request's step, query head); a workgroup holds four such
-// wavefronts that share nothing.  The wavefront walks the keys its rows can see, 64 at a time,
-// from the first key of its first row's window (rounded down to 8, which stays inside that key's
-// page) to its last row's position: the block's keys [64][D] and values [D][64] (as the pages hold
-// them) go through the wavefront's own part of LDS.  Scores are computed transposed (keys as the
+// One workgroup of four wavefronts per (16 rows of one request's step, query head).  The keys
+// the rows can see, from the first key of the first row's window (rounded down to 8, which stays
+// inside that key's page) to the last row's position, are walked in blocks of 64, the wavefronts
+// taking the blocks in turn and adding their sums at the end (a single token with a window of a
+// thousand keys is then four chains of four blocks, not one of sixteen).  A block's keys [64][D]
+// and values [D][64] (as the pages hold them) go through the wavefront's own part of LDS, and are
+// asked for from memory while the block before is multiplied.  Scores are computed transposed (keys as the
 // first operand), so a lane ends up with four neighbouring keys of one row in each of the block's
 // four tiles; two tiles' weights, rounded to bfloat16, are then a lane's second operand of the
 // product with the values as they are, the eight keys dealt to the instruction in the order the
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_
     __bf16* ks = reinterpret_cast<__bf16*>(sa_lds) + static_cast<size_t>(wave) * (SA_KEYS * KROW + D * VROW);
     __bf16* vs = ks + SA_KEYS * KROW;
     // which 16 rows: tiles of all requests of the step, one after the other
-    int tile = blockIdx.x * SA_WAVES + wave, s = 0, row0 = 0, n = 0;
+    int tile = blockIdx.x, s = 0, row0 = 0, n = 0;
     for (; s < n_seqs; ++s) {
         row0 = cu_seqlens[s];
         n = cu_seqlens[s + 1] - row0;
@@ -143,19 +145,22 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_
     for (int dt = 0; dt < DT; ++dt) oacc[dt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
     const int key_first = window > 0 ? max(0, pos0 - window + 1) : 0;
     const size_t head_stride = static_cast<size_t>(page_tokens) * D;
-    for (int kb = key_first & ~7; kb <= pos_last; kb += SA_KEYS) {
-        // stage: keys kb .. kb + 63 (those past pos_last: the last one again), values with zeros past pos_last
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        for (int c = lane; c < SA_KEYS * (D / 8); c += CELEG_WAVE) {
-            const int key_in = c / (D / 8), part = c % (D / 8);
+    constexpr int KCH = SA_KEYS * (D / 8) / CELEG_WAVE, VCH = D * (SA_KEYS / 8) / CELEG_WAVE;   // 16-byte pieces a lane
+    sa_u32x4 kpre[KCH], vpre[VCH];
+    // a block's pieces from memory into registers: keys kb .. kb + 63 (those past pos_last: the last
+    // one again), values with zeros past pos_last
+    auto fetch = [&](int kb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < KCH; ++i) {
+            const int c = lane + CELEG_WAVE * i, key_in = c / (D / 8), part = c % (D / 8);
             const int key = min(kb + key_in, pos_last);
             const bf16* src = k_pool + ((static_cast<size_t>(pages[key / page_tokens]) * n_layers + layer) * kv_heads + kvh) * head_stride +
                               static_cast<size_t>(key % page_tokens) * D + 8 * part;
-            *reinterpret_cast<sa_u32x4*>(ks + key_in * KROW + 8 * part) = *reinterpret_cast<const sa_u32x4*>(src);
+            kpre[i] = *reinterpret_cast<const sa_u32x4*>(src);
         }
-        for (int c = lane; c < D * (SA_KEYS / 8); c += CELEG_WAVE) {
-            const int d = c / (SA_KEYS / 8), part = c % (SA_KEYS / 8);
+#pragma unroll
+        for (int i = 0; i < VCH; ++i) {
+            const int c = lane + CELEG_WAVE * i, d = c / (SA_KEYS / 8), part = c % (SA_KEYS / 8);
             const int key = kb + 8 * part;         // eight keys that lie side by side in one page
             sa_u32x4 val = {0u, 0u, 0u, 0u};
             if (key <= pos_last) {
@@ -170,11 +175,28 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_
                     if (live == 1) val[0] &= 0x0000ffffu;
                 }
             }
-            *reinterpret_cast<sa_u32x4*>(vs + d * VROW + 8 * part) = val;
+            vpre[i] = val;
+        }
+    };
+    const int kb0 = (key_first & ~7) + wave * SA_KEYS;
+    if (kb0 <= pos_last) fetch(kb0);
+    for (int kb = kb0; kb <= pos_last; kb += SA_WAVES * SA_KEYS) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < KCH; ++i) {
+            const int c = lane + CELEG_WAVE * i;
+            *reinterpret_cast<sa_u32x4*>(ks + (c / (D / 8)) * KROW + 8 * (c % (D / 8))) = kpre[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VCH; ++i) {
+            const int c = lane + CELEG_WAVE * i;
+            *reinterpret_cast<sa_u32x4*>(vs + (c / (SA_KEYS / 8)) * VROW + 8 * (c % (SA_KEYS / 8))) = vpre[i];
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (kb + SA_WAVES * SA_KEYS <= pos_last) fetch(kb + SA_WAVES * SA_KEYS);
         // scores, transposed: tile kt holds keys kb + 16 kt + 4 quad + i of row r
         sa_f32x4 sacc[4];
 #pragma unroll
@@ -209,7 +231,24 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_
             }
         }
     }
-    if (r >= rows_here) return;
+    // the wavefronts' sums meet in LDS (every wavefront's staging area is its own again after the
+    // barrier), the first one adds them in the order of the wavefronts and stores
+    __syncthreads();
+    float* sums = reinterpret_cast<float*>(sa_lds);
+    if (wave > 0) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sums[(((wave - 1) * DT + dt) * 4 + i) * CELEG_WAVE + lane] = oacc[dt][i];
+    }
+    __syncthreads();
+    if (wave > 0 || r >= rows_here) return;
+#pragma unroll
+    for (int w = 1; w < SA_WAVES; ++w)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oacc[dt][i] += sums[(((w - 1) * DT + dt) * 4 + i) * CELEG_WAVE + lane];
     const float g = gate ? sa_sigmoid(to_float(gate[static_cast<size_t>(row0 + my_row) * ldg + h])) : 1.0f;
     bf16* orow = out + static_cast<size_t>(row0 + my_row) * ldo + static_cast<size_t>(h) * D;
 #pragma unroll
@@ -257,7 +296,7 @@ extern "C" int celeg_sigmoid_attention_fast(const void* q, int ldq, const void* 
     if (max_tiles <= 0 || n_seqs <= 0) return 0;
     if (!celeg_sigmoid_attention_fast_ok(head_dim) || q_heads % kv_heads || page_tokens % 8 || ldq % 8 || ldo % 4)
         return static_cast<int>(hipErrorInvalidValue);
-    dim3 grid((max_tiles + SA_WAVES - 1) / SA_WAVES, q_heads), block(SA_WAVES * CELEG_WAVE);
+    dim3 grid(max_tiles, q_heads), block(SA_WAVES * CELEG_WAVE);
     const size_t lds = static_cast<size_t>(SA_WAVES) * (SA_KEYS * (head_dim + 8) + head_dim * (SA_KEYS + 8)) * 2;
 #define CELEG_SA_FAST(D_)                                                                                                        \
     hipLaunchKernelGGL(sigmoid_attention_mfma_kernel<D_>, grid, block, lds, stream, static_cast<const bf16*>(q), ldq,               \
