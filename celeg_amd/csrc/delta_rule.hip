@@ -151,6 +151,39 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_kernel(
         for (int d = 0; d < D; ++d) mine[static_cast<size_t>(d) * V + j] = S[d * CELEG_WAVE + lane];
 }
 
+// What two neighbouring rows of a request's step need of each other when the recurrence takes them
+// together: for the rows at even places of their segment (and not its last), per query/key head,
+// k1.k2, k1.q1, k1.q2, k2.q2 (1: the row, 2: the next one).  One wavefront per (row, head).
+__global__ __launch_bounds__(CELEG_WAVE) void delta_pairs_kernel(const float* __restrict__ qk, const int* __restrict__ token_seq,
+                                                                 const int* __restrict__ cu_seqlens, float* __restrict__ pairs, int G,
+                                                                 int D) {
+    const int t = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+    const int seq = token_seq[t], row0 = cu_seqlens[seq], end = cu_seqlens[seq + 1];
+    if (((t - row0) & 1) || t + 1 >= end) return;
+    const float* q1 = qk + static_cast<size_t>(t) * 2 * G * D + static_cast<size_t>(g) * D;
+    const float* k1 = q1 + static_cast<size_t>(G) * D;
+    const float* q2 = q1 + static_cast<size_t>(2) * G * D;
+    const float* k2 = k1 + static_cast<size_t>(2) * G * D;
+    float kk = 0.f, kq1 = 0.f, kq2 = 0.f, k2q2 = 0.f;
+    for (int d = lane; d < D; d += CELEG_WAVE) {
+        kk = fmaf(k1[d], k2[d], kk);
+        kq1 = fmaf(k1[d], q1[d], kq1);
+        kq2 = fmaf(k1[d], q2[d], kq2);
+        k2q2 = fmaf(k2[d], q2[d], k2q2);
+    }
+    kk = wave_sum(kk);
+    kq1 = wave_sum(kq1);
+    kq2 = wave_sum(kq2);
+    k2q2 = wave_sum(k2q2);
+    if (lane == 0) {
+        float* dst = pairs + (static_cast<size_t>(t) * G + g) * 4;
+        dst[0] = kk;
+        dst[1] = kq1;
+        dst[2] = kq2;
+        dst[3] = k2q2;
+    }
+}
+
 // The sum of v over every group of W neighbouring lanes (1 to 16), in all of them, by the vector
 // unit's cross-lane modifiers: lanes swapped in pairs and in pairs of pairs, then the halves of 8
 // and of 16 mirrored.  Both sides of every exchange add the same two numbers, so the lanes agree.
@@ -166,21 +199,23 @@ __device__ __forceinline__ float lanes_sum(float v) {
     return v;
 }
 
-// The same recurrence with S in registers, for dim = 16 * DL: DL neighbouring lanes share a column
-// of S, each holding 16 of its values, so a wavefront owns 64 / DL columns and the sums over dim
-// meet by log2(DL) exchanges between neighbours.  The rows of a request are taken in blocks of TB
+// The same recurrence with S in registers, for dim = DL * DPL: DL neighbouring lanes share a column
+// of S, each holding DPL of its values, so a wavefront owns 64 / DL columns and the sums over dim
+// meet by log2(DL) exchanges between neighbours.  (Few values a lane: a token's passes over the
+// state are short, and it is their chain from token to token that the kernel's time is.)  The rows of a request are taken in blocks of TB
 // tokens: a block's q, k, write strengths and decays are staged in LDS (asked for from memory while
 // the block before is computed), its values sit in registers.  With u = beta (v - a (S^T k)) the
 // new column is a S + k u, read out with q in the same pass.
-template <int DL>
+template <int DL, int DPL>
 __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
     const float* __restrict__ qk, const float* __restrict__ v, const float* __restrict__ beta_decay, float* __restrict__ state,
-    size_t state_stride, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot, float* __restrict__ out, int G, int H,
-    int V) {
-    constexpr int D = 16 * DL, CPW = CELEG_WAVE / DL, TB = D <= 64 ? 16 : 8, ROW = 2 * D, PER_LANE = TB * ROW / CELEG_WAVE;
+    size_t state_stride, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot, float* __restrict__ out,
+    const float* __restrict__ pairs, int G, int H, int V) {
+    constexpr int D = DPL * DL, NC = DPL / 4, CPW = CELEG_WAVE / DL, TB = D <= 64 ? 16 : 8, ROW = 2 * D, PER_LANE = TB * ROW / CELEG_WAVE;
     typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ __attribute__((aligned(16))) float qk_s[TB * ROW];
     __shared__ float bd_s[TB * 2];
+    __shared__ float pair_s[TB * 2];
     const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int sub = lane % DL, j = blockIdx.z * CPW + lane / DL;
     const bool live = j < V;
@@ -189,11 +224,11 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
     const int row0 = cu_seqlens[s], n = cu_seqlens[s + 1] - row0;
     if (n <= 0) return;
     float* mine = state + static_cast<size_t>(seq_slot[s]) * state_stride + static_cast<size_t>(h) * D * V;
-    float S[16];
+    float S[DPL];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) S[i] = mine[static_cast<size_t>(sub * 16 + i) * V + jj];
+    for (int i = 0; i < DPL; ++i) S[i] = mine[static_cast<size_t>(sub * DPL + i) * V + jj];
     const size_t ldqk = static_cast<size_t>(2) * G * D;
-    float pre[PER_LANE], pre_v[TB], pre_bd = 0.f;
+    float pre[PER_LANE], pre_v[TB], pre_bd = 0.f, pre_pair = 0.f;
     auto fetch = [&](int block) __attribute__((always_inline)) {
         const int t0 = block * TB;
 #pragma unroll
@@ -205,6 +240,8 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
 #pragma unroll
         for (int tt = 0; tt < TB; ++tt) pre_v[tt] = v[static_cast<size_t>(row0 + min(t0 + tt, n - 1)) * H * V + static_cast<size_t>(h) * V + jj];
         if (lane < 2 * TB) pre_bd = beta_decay[static_cast<size_t>(row0 + min(t0 + lane / 2, n - 1)) * 2 * H + (lane & 1) * H + h];
+        // (what the pairs of a whole block need; a block that is not whole goes token by token)
+        if (pairs && lane < 2 * TB && t0 + TB <= n) pre_pair = pairs[(static_cast<size_t>(row0 + t0 + 2 * (lane >> 2)) * G + g) * 4 + (lane & 3)];
     };
     fetch(0);
     const int n_blocks = (n + TB - 1) / TB;
@@ -212,34 +249,35 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < PER_LANE; ++i) qk_s[lane + CELEG_WAVE * i] = pre[i];
-        if (lane < 2 * TB) bd_s[lane] = pre_bd;
+        if (lane < 2 * TB) {
+            bd_s[lane] = pre_bd;
+            pair_s[lane] = pre_pair;
+        }
         float vals[TB];
 #pragma unroll
         for (int tt = 0; tt < TB; ++tt) vals[tt] = pre_v[tt];
         __syncthreads();
         if (block + 1 < n_blocks) fetch(block + 1);
         const int count = min(TB, n - block * TB);
+        auto token = [&](int tt, float value) __attribute__((always_inline)) {
+            const float* qrow = qk_s + tt * ROW + sub * DPL;
+            f4 q4[NC], k4[NC];
 #pragma unroll
-        for (int tt = 0; tt < TB; ++tt) {
-            if (tt >= count) break;
-            const float* qrow = qk_s + tt * ROW + sub * 16;
-            f4 q4[4], k4[4];
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
+            for (int c = 0; c < NC; ++c) {
                 q4[c] = *reinterpret_cast<const f4*>(qrow + 4 * c);
                 k4[c] = *reinterpret_cast<const f4*>(qrow + D + 4 * c);
             }
             const float beta = bd_s[2 * tt], decay = bd_s[2 * tt + 1];
             float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
+            for (int c = 0; c < NC; ++c)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) part[e] = fmaf(k4[c][e], S[4 * c + e], part[e]);
             const float kv = lanes_sum<DL>((part[0] + part[1]) + (part[2] + part[3]));
-            const float u = beta * (vals[tt] - decay * kv);
+            const float u = beta * (value - decay * kv);
             float opart[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
+            for (int c = 0; c < NC; ++c)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const float sd = fmaf(k4[c][e], u, decay * S[4 * c + e]);
@@ -248,11 +286,72 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
                 }
             const float o = lanes_sum<DL>((opart[0] + opart[1]) + (opart[2] + opart[3]));
             if (live && sub == 0) out[static_cast<size_t>(row0 + block * TB + tt) * H * V + static_cast<size_t>(h) * V + j] = o;
+        };
+        // Two tokens together: with p = S^T k and r = S^T q of both tokens against the state before
+        // them (one pass over S), u1 = b1 (v1 - a1 p1), u2 = b2 (v2 - a2 (a1 p2 + u1 k1.k2)),
+        // o1 = a1 r1 + u1 k1.q1, o2 = a2 (a1 r2 + u1 k1.q2) + u2 k2.q2, and the state after them is
+        // a2 a1 S + a2 u1 k1 + u2 k2 (a second pass): half as many passes that wait for one another.
+        auto two_tokens = [&](int tt, float v1, float v2) __attribute__((always_inline)) {
+            const float* row1 = qk_s + tt * ROW + sub * DPL;
+            const float* row2 = row1 + ROW;
+            f4 q1[NC], k1[NC], q2[NC], k2[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                q1[c] = *reinterpret_cast<const f4*>(row1 + 4 * c);
+                k1[c] = *reinterpret_cast<const f4*>(row1 + D + 4 * c);
+                q2[c] = *reinterpret_cast<const f4*>(row2 + 4 * c);
+                k2[c] = *reinterpret_cast<const f4*>(row2 + D + 4 * c);
+            }
+            const float b1 = bd_s[2 * tt], a1 = bd_s[2 * tt + 1], b2 = bd_s[2 * tt + 2], a2 = bd_s[2 * tt + 3];
+            const float* ps = pair_s + 2 * tt;
+            const float k1k2 = ps[0], k1q1 = ps[1], k1q2 = ps[2], k2q2 = ps[3];
+            float p1[2] = {0.f, 0.f}, p2[2] = {0.f, 0.f}, r1[2] = {0.f, 0.f}, r2[2] = {0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float sv = S[4 * c + e];
+                    p1[e & 1] = fmaf(k1[c][e], sv, p1[e & 1]);
+                    p2[e & 1] = fmaf(k2[c][e], sv, p2[e & 1]);
+                    r1[e & 1] = fmaf(q1[c][e], sv, r1[e & 1]);
+                    r2[e & 1] = fmaf(q2[c][e], sv, r2[e & 1]);
+                }
+            const float sp1 = lanes_sum<DL>(p1[0] + p1[1]), sp2 = lanes_sum<DL>(p2[0] + p2[1]);
+            const float sr1 = lanes_sum<DL>(r1[0] + r1[1]), sr2 = lanes_sum<DL>(r2[0] + r2[1]);
+            const float u1 = b1 * (v1 - a1 * sp1);
+            const float u2 = b2 * (v2 - a2 * fmaf(u1, k1k2, a1 * sp2));
+            const float o1 = fmaf(u1, k1q1, a1 * sr1);
+            const float o2 = fmaf(u2, k2q2, a2 * fmaf(u1, k1q2, a1 * sr2));
+            const float both = a2 * a1, first = a2 * u1;
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) S[4 * c + e] = fmaf(k2[c][e], u2, fmaf(k1[c][e], first, both * S[4 * c + e]));
+            if (live && sub == 0) {
+                float* dst = out + static_cast<size_t>(row0 + block * TB + tt) * H * V + static_cast<size_t>(h) * V + j;
+                dst[0] = o1;
+                dst[static_cast<size_t>(H) * V] = o2;
+            }
+        };
+        if (count == TB && pairs) {
+            // a whole block: one run of instructions, so that the next tokens' operands are read while
+            // these are computed
+#pragma unroll
+            for (int tt = 0; tt < TB; tt += 2) two_tokens(tt, vals[tt], vals[tt + 1]);
+        } else if (count == TB) {
+#pragma unroll
+            for (int tt = 0; tt < TB; ++tt) token(tt, vals[tt]);
+        } else {
+#pragma unroll
+            for (int tt = 0; tt < TB; ++tt) {
+                if (tt >= count) break;
+                token(tt, vals[tt]);
+            }
         }
     }
     if (live)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mine[static_cast<size_t>(sub * 16 + i) * V + j] = S[i];
+        for (int i = 0; i < DPL; ++i) mine[static_cast<size_t>(sub * DPL + i) * V + j] = S[i];
 }
 
 // one wavefront per (row, head): out = o / sqrt(mean(o^2) + eps) * w * silu(gate)
@@ -308,20 +407,26 @@ extern "C" int celeg_delta_conv_state(const void* proj, int ld, int dtype, float
 
 extern "C" int celeg_delta_scan(const float* qk, const float* v, const float* beta_decay, float* state, size_t state_stride,
                                 const int* cu_seqlens, const int* seq_slot, float* out, int n_seqs, int G, int H, int D, int V,
-                                int general, hipStream_t stream) {
+                                int general, const int* token_seq, float* pairs, int n_tokens, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     if (H % G) return static_cast<int>(hipErrorInvalidValue);
     if (!general && (D == 16 || D == 32 || D == 64 || D == 128 || D == 256)) {
-        const int DL = D / 16, cpw = CELEG_WAVE / DL;
+        const int DL = D == 16 ? 4 : D == 32 ? 8 : 16, cpw = CELEG_WAVE / DL;
         dim3 grid(n_seqs, H, (V + cpw - 1) / cpw), block(CELEG_WAVE);
-#define CELEG_DELTA_REG(DL_)                                                                                                  \
-    hipLaunchKernelGGL(delta_scan_reg_kernel<DL_>, grid, block, 0, stream, qk, v, beta_decay, state, state_stride, cu_seqlens, \
-                       seq_slot, out, G, H, V)
-        if (DL == 1) CELEG_DELTA_REG(1);
-        else if (DL == 2) CELEG_DELTA_REG(2);
-        else if (DL == 4) CELEG_DELTA_REG(4);
-        else if (DL == 8) CELEG_DELTA_REG(8);
-        else CELEG_DELTA_REG(16);
+        // pairs (room for n_tokens * G * 4 floats, or null): steps with rows to pair take two tokens together
+        if (pairs && n_tokens > n_seqs) {
+            hipLaunchKernelGGL(delta_pairs_kernel, dim3(n_tokens, G), dim3(CELEG_WAVE), 0, stream, qk, token_seq, cu_seqlens, pairs, G, D);
+        } else {
+            pairs = nullptr;
+        }
+#define CELEG_DELTA_REG(DL_, DPL_)                                                                                                  \
+    hipLaunchKernelGGL((delta_scan_reg_kernel<DL_, DPL_>), grid, block, 0, stream, qk, v, beta_decay, state, state_stride, cu_seqlens, \
+                       seq_slot, out, pairs, G, H, V)
+        if (D == 16) CELEG_DELTA_REG(4, 4);
+        else if (D == 32) CELEG_DELTA_REG(8, 4);
+        else if (D == 64) CELEG_DELTA_REG(16, 4);
+        else if (D == 128) CELEG_DELTA_REG(16, 8);
+        else CELEG_DELTA_REG(16, 16);
 #undef CELEG_DELTA_REG
         return CELEG_LAUNCH_RESULT();
     }

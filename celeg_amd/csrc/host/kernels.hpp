@@ -167,7 +167,7 @@ int celeg_delta_conv_state(const void* proj, int ld, int dtype, float* conv_stat
                            const int* seq_slot, int n_seqs, int n_channels, int taps, hipStream_t stream);
 int celeg_delta_scan(const float* qk, const float* v, const float* beta_decay, float* state, size_t state_stride,
                      const int* cu_seqlens, const int* seq_slot, float* out, int n_seqs, int G, int H, int D, int V,
-                     int general, hipStream_t stream);
+                     int general, const int* token_seq, float* pairs, int n_tokens, hipStream_t stream);
 int celeg_delta_gated_norm(const float* o, const float* w, const void* gate, int ldg, int dtype, float eps, void* out,
                            int n_tokens, int H, int V, hipStream_t stream);
 }

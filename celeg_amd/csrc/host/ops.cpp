@@ -819,7 +819,7 @@ void Ops::delta_prepare(const Tensor& proj, int col_b, int col_a, const DeltaSha
 }
 
 void Ops::delta_scan(const Tensor& qk, const Tensor& v, const Tensor& beta_decay, const Tensor& state, const Tensor& out,
-                     const DeltaShape& s, const StepBatch& batch) {
+                     const DeltaShape& s, const StepBatch& batch, Workspace& ws) {
     dev(qk, "qk", DType::F32);
     dev(v, "v", DType::F32);
     dev(beta_decay, "beta_decay", DType::F32);
@@ -831,9 +831,14 @@ void Ops::delta_scan(const Tensor& qk, const Tensor& v, const Tensor& beta_decay
     need(state.ndim >= 2 && state.numel() / state.shape[0] == per_slot && state.stride[state.ndim - 1] == 1,
          "delta_scan: state must be [slots, heads, dim, vdim]");
     need(s.dim <= 256 && (s.dim <= 248 || s.dim == 256), "delta_scan: dim " + std::to_string(s.dim) + " exceeds 256");
+    // rows that have a neighbour in their request's step are taken two at a time
+    float* pairs = nullptr;
+    if (delta_pairs && !delta_general && batch.n_tokens > batch.n_seqs)
+        pairs = ws.buf("delta_pairs", DType::F32, {T, 4LL * s.kv_heads}).as<float>();
     kernel_check(celeg_delta_scan(qk.as<float>(), v.as<float>(), beta_decay.as<float>(), state.as<float>(),
                                   static_cast<size_t>(state.stride[0]), batch.cu_seqlens, batch.seq_slot, out.as<float>(), batch.n_seqs,
-                                  s.kv_heads, s.heads, s.dim, s.vdim, delta_general ? 1 : 0, stream), "delta_scan");
+                                  s.kv_heads, s.heads, s.dim, s.vdim, delta_general ? 1 : 0, batch.token_seq, pairs, batch.n_tokens, stream),
+                 "delta_scan");
 }
 
 void Ops::delta_gated_norm(const Tensor& o, const Tensor& weight, const Tensor& gate, float eps, const Tensor& out, int heads, int vdim) {

@@ -124,6 +124,7 @@ public:
     bool decode_whole(long long groups, int rounds) const;
     bool attention_general = false;      // always the general attention kernel
     bool delta_general = false;          // the delta rule's recurrence always by the kernel for any dim
+    bool delta_pairs = true;             // the recurrence in registers takes whole blocks of rows two tokens at a time
     bool use_sigmoid_mfma = true;        // bfloat16 attention with sigmoid weights on the matrix cores
     bool use_router_kernel = true;       // the router's product inside the routing kernel
     bool use_moe_mfma = true;            // bfloat16 products of routed experts and per-head matrices on the matrix cores
@@ -198,7 +199,7 @@ public:
                        const StepBatch& batch);
     // the recurrence over the step's rows of every request, from and into state [slots, heads, dim, vdim]
     void delta_scan(const Tensor& qk, const Tensor& v, const Tensor& beta_decay, const Tensor& state, const Tensor& out,
-                    const DeltaShape& shape, const StepBatch& batch);
+                    const DeltaShape& shape, const StepBatch& batch, Workspace& ws);
     // out = o / rms(o) * weight * silu(gate) per head; o [rows, heads * vdim] 32-bit, gate a view with dense rows
     void delta_gated_norm(const Tensor& o, const Tensor& weight, const Tensor& gate, float eps, const Tensor& out, int heads, int vdim);
     // whether a decode-only step's attention can prepare and write the step's own keys and values itself

@@ -1323,7 +1323,7 @@ public:
         rt.ops.delta_prepare(proj, static_cast<int>(col_b_), static_cast<int>(col_a_), shape_, conv_w_->view, a_log_->view,
                              dt_bias_->view, cache.states.at("conv"), qk, v, beta_decay, batch);
         Tensor o = rt.ws.buf("delta_o", DType::F32, {T, v_width()});
-        rt.ops.delta_scan(qk, v, beta_decay, cache.states.at("S"), o, shape_, batch);
+        rt.ops.delta_scan(qk, v, beta_decay, cache.states.at("S"), o, shape_, batch, rt.ws);
         Tensor gated = rt.ws.buf("delta_gated", rt.dtype, {T, v_width()});
         rt.ops.delta_gated_norm(o, norm_->view, proj.cols(col_gate_, v_width()), eps_, gated, shape_.heads, shape_.vdim);
         Tensor out = rt.ws.buf("mixer_out", rt.dtype, {T, width_});

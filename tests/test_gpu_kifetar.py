@@ -163,8 +163,9 @@ def test_engine_matches_plain(folders, name, dtype, mode):
 
 
 def test_batches_of_unequal_requests_equal_each_alone(folders):
-    """In 32-bit a row's logits are the same numbers whatever else is in the batch and however
-    the prompt was cut (every kernel's order of additions depends on the row alone)."""
+    """In 32-bit a row's logits do not depend on what else is in the batch or on how the prompt was
+    cut, beyond the rounding of 32-bit sums taken in another order (the delta rule takes the rows of
+    a whole block two at a time, a cut block one at a time): held to 2e-5 of the largest logit."""
     folder = folders("K1", "float32")
     reqs = requests_of("K1")
     alone_steps, mixed_steps = whole_schedule(reqs), mixed_schedule(reqs, seed=3)
@@ -173,7 +174,7 @@ def test_batches_of_unequal_requests_equal_each_alone(folders):
     lm2, _ = load(folder, "float32", mixed_steps)
     mixed = EngineDriver(lm2).run(mixed_steps)
     for rid in reqs:
-        assert torch.equal(alone[rid], mixed[rid]), rid
+        assert float((alone[rid] - mixed[rid]).abs().max()) <= 2e-5 * float(alone[rid].abs().max()), rid
 
 
 # ------------------------------------------------------------------ weights made so that a fault shows
