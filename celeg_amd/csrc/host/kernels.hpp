@@ -153,7 +153,7 @@ int celeg_sigmoid_attention(const void* q, int ldq, const void* k_pool, const vo
                             int kv_heads, int head_dim, int page_tokens, int n_layers, int layer, float scale, int window,
                             hipStream_t stream);
 int celeg_sigmoid_attention_fast_ok(int head_dim);
-int celeg_sigmoid_attention_fast(const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
+int celeg_sigmoid_attention_fast(int form, const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
                                  int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start, int n_seqs,
                                  int max_tiles, const float* temp, const float* bias, const void* gate, int ldg, void* out,
                                  int ldo, int q_heads, int kv_heads, int head_dim, int page_tokens, int n_layers, int layer,

@@ -766,10 +766,13 @@ void Ops::sigmoid_attention(const Tensor& q, const Tensor& out, int heads, int k
     if (q.dtype == DType::BF16 && use_sigmoid_mfma && !attention_general && celeg_sigmoid_attention_fast_ok(head_dim) &&
         kv.page_tokens >= 8 && (kv.page_tokens & (kv.page_tokens - 1)) == 0 && ldq % 8 == 0 && head_dim % 8 == 0 &&
         (reinterpret_cast<uintptr_t>(q.data) & 15) == 0) {
-        // tiles of 16 rows: at most one partly filled tile per request
-        const int max_tiles = static_cast<int>(T) / 16 + batch.n_seqs;
+        // portions of prompts: tiles of 64 rows that share their staged keys; single tokens and short
+        // portions: tiles of 16 rows whose key blocks the wavefronts take in turn.  At most one
+        // partly filled tile per request.
+        const int form = sigmoid_rows_form >= 0 ? sigmoid_rows_form : (batch.max_seg_len > 16 ? 1 : 0);
+        const int max_tiles = static_cast<int>(T) / (form == 1 ? 64 : 16) + batch.n_seqs;
         took(batch.decode_only ? Path::AttentionSigmoidDecode : Path::AttentionSigmoidRows);
-        kernel_check(celeg_sigmoid_attention_fast(q.data, ldq, kv.k, kv.v, kv.table, kv.table_stride, batch.cu_seqlens, batch.seq_slot,
+        kernel_check(celeg_sigmoid_attention_fast(form, q.data, ldq, kv.k, kv.v, kv.table, kv.table_stride, batch.cu_seqlens, batch.seq_slot,
                                                   batch.seq_start, batch.n_seqs, max_tiles, temp ? temp->as<float>() : nullptr,
                                                   bias ? bias->as<float>() : nullptr, gate ? gate->data : nullptr, ldg, out.data,
                                                   static_cast<int>(qw), heads, kv_heads, head_dim, kv.page_tokens, kv.n_layers, kv.layer,

@@ -126,6 +126,7 @@ public:
     bool delta_general = false;          // the delta rule's recurrence always by the kernel for any dim
     bool delta_pairs = true;             // the recurrence in registers takes whole blocks of rows two tokens at a time
     bool use_sigmoid_mfma = true;        // bfloat16 attention with sigmoid weights on the matrix cores
+    int sigmoid_rows_form = -1;          // -1: by the step's longest portion; 0 tiles of 16 rows, 1 tiles of 64 rows
     bool use_router_kernel = true;       // the router's product inside the routing kernel
     bool use_moe_mfma = true;            // bfloat16 products of routed experts and per-head matrices on the matrix cores
     bool use_latent_mfma = true;         // bfloat16 attention over a latent cache on the matrix cores

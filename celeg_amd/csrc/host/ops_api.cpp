@@ -160,6 +160,7 @@ void set_knobs(Ops& ops, const Json& knobs) {
         else if (name == "use_rope_table") ops.use_rope_table = v != 0;
         else if (name == "delta_general") ops.delta_general = v != 0;
         else if (name == "delta_pairs") ops.delta_pairs = v != 0;
+        else if (name == "sigmoid_rows_form") ops.sigmoid_rows_form = static_cast<int>(v);
         else if (name == "use_sigmoid_mfma") ops.use_sigmoid_mfma = v != 0;
         else if (name == "use_argmax_parts") ops.use_argmax_parts = v != 0;
         else if (name == "use_head_argmax") ops.use_head_argmax = v != 0;

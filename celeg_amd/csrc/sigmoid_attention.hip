@@ -259,6 +259,145 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_
     }
 }
 
+// The form for portions of prompts: a workgroup per (64 rows of one request's step, query head),
+// 16 rows a wavefront.  The tile's key blocks are staged once for all four wavefronts, by all of
+// them, into one of two buffers in turn (the next block is asked for from memory while this one
+// is multiplied, and one barrier a block is enough: a buffer is written again only after every
+// wavefront has passed the barrier behind the block that read it).  A wavefront leaves out the
+// blocks none of its rows can see.  The arithmetic is the single-tile form's.
+template <int D>
+__global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_rows_kernel(
+    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
+    const int* __restrict__ table, int table_stride, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_start, int n_seqs, const float* __restrict__ temp, const float* __restrict__ bias,
+    const bf16* __restrict__ gate, int ldg, bf16* __restrict__ out, int ldo, int q_heads, int kv_heads, int page_tokens,
+    int n_layers, int layer, float scale, int window) {
+    constexpr int KROW = D + 8, VROW = SA_KEYS + 8, KS = D / 32, DT = D / 16, BUF = SA_KEYS * KROW + D * VROW;
+    constexpr int THREADS = SA_WAVES * CELEG_WAVE, KCH = SA_KEYS * (D / 8) / THREADS, VCH = D * (SA_KEYS / 8) / THREADS;
+    extern __shared__ __attribute__((aligned(16))) unsigned char sa_lds[];
+    __bf16* lds = reinterpret_cast<__bf16*>(sa_lds);
+    const int wave = threadIdx.x / CELEG_WAVE, lane = threadIdx.x % CELEG_WAVE, tid = threadIdx.x;
+    int tile = blockIdx.x, s = 0, row0 = 0, n = 0;
+    for (; s < n_seqs; ++s) {
+        row0 = cu_seqlens[s];
+        n = cu_seqlens[s + 1] - row0;
+        const int tiles = (n + 63) / 64;
+        if (tile < tiles) break;
+        tile -= tiles;
+    }
+    if (s >= n_seqs) return;
+    const int h = blockIdx.y, kvh = h / (q_heads / kv_heads);
+    const int r = lane & 15, quad = lane >> 4;
+    const int tile_row = tile * 64, tile_rows = min(64, n - tile_row);
+    const int tile_pos0 = seq_start[s] + tile_row, pos_last = tile_pos0 + tile_rows - 1;
+    const int first_row = tile_row + 16 * wave, rows_here = min(16, n - first_row);      // <= 0: this wavefront only stages
+    const int my_row = first_row + max(0, min(r, rows_here - 1));
+    const int safe_row = min(my_row, n - 1);
+    const int my_pos = seq_start[s] + safe_row;
+    const int wave_pos0 = seq_start[s] + first_row, wave_last = wave_pos0 + rows_here - 1;
+    const int* pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
+    const float tau = scale * (temp ? temp[h] : 1.0f), beta = bias ? bias[h] : 0.0f;
+    sa_bf16x8 qreg[KS];
+    const bf16* qrow = q + static_cast<size_t>(row0 + safe_row) * ldq + static_cast<size_t>(h) * D;
+#pragma unroll
+    for (int st = 0; st < KS; ++st) qreg[st] = __builtin_bit_cast(sa_bf16x8, *reinterpret_cast<const sa_u32x4*>(qrow + 32 * st + 8 * quad));
+    sa_f32x4 oacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
+    const int key_first = window > 0 ? max(0, tile_pos0 - window + 1) : 0;
+    const size_t head_stride = static_cast<size_t>(page_tokens) * D;
+    sa_u32x4 kpre[KCH], vpre[VCH];
+    auto fetch = [&](int kb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < KCH; ++i) {
+            const int c = tid + THREADS * i, key_in = c / (D / 8), part = c % (D / 8);
+            const int key = min(kb + key_in, pos_last);
+            const bf16* src = k_pool + ((static_cast<size_t>(pages[key / page_tokens]) * n_layers + layer) * kv_heads + kvh) * head_stride +
+                              static_cast<size_t>(key % page_tokens) * D + 8 * part;
+            kpre[i] = *reinterpret_cast<const sa_u32x4*>(src);
+        }
+#pragma unroll
+        for (int i = 0; i < VCH; ++i) {
+            const int c = tid + THREADS * i, d = c / (SA_KEYS / 8), part = c % (SA_KEYS / 8);
+            const int key = kb + 8 * part;
+            sa_u32x4 val = {0u, 0u, 0u, 0u};
+            if (key <= pos_last) {
+                const bf16* src = v_pool + ((static_cast<size_t>(pages[key / page_tokens]) * n_layers + layer) * kv_heads + kvh) * head_stride +
+                                  static_cast<size_t>(d) * page_tokens + key % page_tokens;
+                val = *reinterpret_cast<const sa_u32x4*>(src);
+                const int live = pos_last - key + 1;
+                if (live < 8) {
+                    if (live <= 6) val[3] = 0u; else val[3] &= 0x0000ffffu;
+                    if (live <= 4) val[2] = 0u; else if (live == 5) val[2] &= 0x0000ffffu;
+                    if (live <= 2) val[1] = 0u; else if (live == 3) val[1] &= 0x0000ffffu;
+                    if (live == 1) val[0] &= 0x0000ffffu;
+                }
+            }
+            vpre[i] = val;
+        }
+    };
+    const int kb0 = key_first & ~7;
+    fetch(kb0);
+    int turn = 0;
+    for (int kb = kb0; kb <= pos_last; kb += SA_KEYS, turn ^= 1) {
+        __bf16* ks = lds + turn * BUF;
+        __bf16* vs = ks + SA_KEYS * KROW;
+#pragma unroll
+        for (int i = 0; i < KCH; ++i) {
+            const int c = tid + THREADS * i;
+            *reinterpret_cast<sa_u32x4*>(ks + (c / (D / 8)) * KROW + 8 * (c % (D / 8))) = kpre[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VCH; ++i) {
+            const int c = tid + THREADS * i;
+            *reinterpret_cast<sa_u32x4*>(vs + (c / (SA_KEYS / 8)) * VROW + 8 * (c % (SA_KEYS / 8))) = vpre[i];
+        }
+        __syncthreads();
+        if (kb + SA_KEYS <= pos_last) fetch(kb + SA_KEYS);
+        // blocks none of this wavefront's rows can see
+        if (rows_here <= 0 || kb > wave_last || (window > 0 && kb + SA_KEYS - 1 < wave_pos0 - window + 1)) continue;
+        sa_f32x4 sacc[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            sacc[kt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int st = 0; st < KS; ++st) {
+                const sa_bf16x8 kf = __builtin_bit_cast(sa_bf16x8, *reinterpret_cast<const sa_u32x4*>(ks + (16 * kt + r) * KROW + 32 * st + 8 * quad));
+                sacc[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qreg[st], sacc[kt], 0, 0, 0);
+            }
+        }
+        sa_bf16x4 w[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kb + 16 * kt + 4 * quad + i;
+                const bool seen = key <= my_pos && (window <= 0 || key > my_pos - window);
+                w[kt][i] = static_cast<__bf16>(seen ? sa_sigmoid(sacc[kt][i] * tau + beta) : 0.0f);
+            }
+#pragma unroll
+        for (int pair = 0; pair < 2; ++pair) {
+            const sa_bf16x8 pw = __builtin_shufflevector(w[2 * pair], w[2 * pair + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const __bf16* vrow = vs + (16 * dt + r) * VROW + 32 * pair + 4 * quad;
+                const sa_u32x2 lo = *reinterpret_cast<const sa_u32x2*>(vrow), hi = *reinterpret_cast<const sa_u32x2*>(vrow + 16);
+                const sa_bf16x8 vf = __builtin_bit_cast(sa_bf16x8, sa_u32x4{lo[0], lo[1], hi[0], hi[1]});
+                oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pw, oacc[dt], 0, 0, 0);
+            }
+        }
+    }
+    if (r >= rows_here) return;
+    const float g = gate ? sa_sigmoid(to_float(gate[static_cast<size_t>(row0 + my_row) * ldg + h])) : 1.0f;
+    bf16* orow = out + static_cast<size_t>(row0 + my_row) * ldo + static_cast<size_t>(h) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const sa_bf16x4 o4 = {static_cast<__bf16>(oacc[dt][0] * g), static_cast<__bf16>(oacc[dt][1] * g),
+                              static_cast<__bf16>(oacc[dt][2] * g), static_cast<__bf16>(oacc[dt][3] * g)};
+        *reinterpret_cast<sa_bf16x4*>(orow + 16 * dt + 4 * quad) = o4;
+    }
+}
+
 }  // namespace
 
 extern "C" int celeg_sigmoid_attention(const void* q, int ldq, const void* k_pool, const void* v_pool, int dtype,
@@ -286,9 +425,11 @@ extern "C" int celeg_sigmoid_attention(const void* q, int ldq, const void* k_poo
 // head sizes the matrix-core kernel takes
 extern "C" int celeg_sigmoid_attention_fast_ok(int head_dim) { return head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128; }
 
-// bfloat16 on the matrix cores; max_tiles: an upper bound on the step's tiles of 16 rows
-// (sum over requests of ceil(rows / 16)); pages of a power of two of at least 8 tokens
-extern "C" int celeg_sigmoid_attention_fast(const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
+// bfloat16 on the matrix cores; form 0: tiles of 16 rows whose key blocks the wavefronts share out
+// (single tokens, short portions), form 1: tiles of 64 rows that stage a key block once for four
+// wavefronts (portions of prompts); max_tiles: an upper bound on the step's tiles (sum over
+// requests of ceil(rows / 16 or 64)); pages of a power of two of at least 8 tokens
+extern "C" int celeg_sigmoid_attention_fast(int form, const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
                                             int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start,
                                             int n_seqs, int max_tiles, const float* temp, const float* bias, const void* gate,
                                             int ldg, void* out, int ldo, int q_heads, int kv_heads, int head_dim, int page_tokens,
@@ -297,9 +438,9 @@ extern "C" int celeg_sigmoid_attention_fast(const void* q, int ldq, const void* 
     if (!celeg_sigmoid_attention_fast_ok(head_dim) || q_heads % kv_heads || page_tokens % 8 || ldq % 8 || ldo % 4)
         return static_cast<int>(hipErrorInvalidValue);
     dim3 grid(max_tiles, q_heads), block(SA_WAVES * CELEG_WAVE);
-    const size_t lds = static_cast<size_t>(SA_WAVES) * (SA_KEYS * (head_dim + 8) + head_dim * (SA_KEYS + 8)) * 2;
+    const size_t lds = static_cast<size_t>(form == 1 ? 2 : SA_WAVES) * (SA_KEYS * (head_dim + 8) + head_dim * (SA_KEYS + 8)) * 2;
 #define CELEG_SA_FAST(D_)                                                                                                        \
-    hipLaunchKernelGGL(sigmoid_attention_mfma_kernel<D_>, grid, block, lds, stream, static_cast<const bf16*>(q), ldq,               \
+    hipLaunchKernelGGL(form == 1 ? sigmoid_attention_rows_kernel<D_> : sigmoid_attention_mfma_kernel<D_>, grid, block, lds, stream, static_cast<const bf16*>(q), ldq,               \
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table, table_stride, cu_seqlens, seq_slot, \
                        seq_start, n_seqs, temp, bias, static_cast<const bf16*>(gate), ldg, static_cast<bf16*>(out), ldo, q_heads,    \
                        kv_heads, page_tokens, n_layers, layer, scale, window)

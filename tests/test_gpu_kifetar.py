@@ -242,15 +242,21 @@ def test_matrix_core_attention_equals_the_general_kernel(tmp_path, dim):
     for steps in (whole_schedule(reqs), tail_decode_schedule(reqs, tail=15), portions_schedule(reqs, sizes=(15, 2, 17, 1, 130, 3, 16, 64)),
                   mixed_schedule(reqs, seed=2, decode_tail=5)):
         got = {}
-        for fast in (1, 0):
+        # the kernel that scores key by key; the form chosen by the step's longest portion; tiles of 16
+        # rows whose key blocks the wavefronts take in turn; tiles of 64 rows that share staged keys
+        for form in ("general", -1, 0, 1):
             lm, _ = load(folder, "bfloat16", steps)
-            lm.set_knob("use_sigmoid_mfma", fast)
-            got[fast] = EngineDriver(lm).run(steps)
-            assert (lm.paths()["attention_sigmoid_rows"] > 0) == bool(fast)
-        for rid in reqs:
-            a, b = got[1][rid].double(), got[0][rid].double()
-            rel = float((a - b).pow(2).mean().sqrt() / b.pow(2).mean().sqrt())
-            assert rel <= 1.5e-2, f"head size {dim}, {rid}: rel rms {rel:.3e}"
+            if form == "general":
+                lm.set_knob("use_sigmoid_mfma", 0)
+            else:
+                lm.set_knob("sigmoid_rows_form", form)
+            got[form] = EngineDriver(lm).run(steps)
+            assert (lm.paths()["attention_sigmoid_rows"] > 0) == (form != "general")
+        for form in (-1, 0, 1):
+            for rid in reqs:
+                a, b = got[form][rid].double(), got["general"][rid].double()
+                rel = float((a - b).pow(2).mean().sqrt() / b.pow(2).mean().sqrt())
+                assert rel <= 1.5e-2, f"head size {dim}, form {form}, {rid}: rel rms {rel:.3e}"
 
 
 def test_delta_rule_in_registers_equals_the_general_kernel(folders):
