@@ -21,6 +21,10 @@ __device__ __forceinline__ size_t sa_cache_offset(int page, int n_layers, int la
 
 __device__ __forceinline__ float sa_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 
+// 1 / (1 + 2^x) by the hardware's exponential and reciprocal (the matrix-core kernels round the weight
+// to bfloat16 right after): 0 for large x, 1 for very negative x
+__device__ __forceinline__ float sa_sigmoid2(float x) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x)); }
+
 #define SA_MAX_DIM_CHUNKS 4  // head_dim <= 256
 
 template <typename T>
@@ -134,7 +138,8 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_
     const int my_row = first_row + min(r, rows_here - 1);      // rows past the end repeat the last one (not stored)
     const int my_pos = seq_start[s] + my_row;
     const int* pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
-    const float tau = scale * (temp ? temp[h] : 1.0f), beta = bias ? bias[h] : 0.0f;
+    // (sigmoid(x) = 1 / (1 + 2^(-x log2 e)): the factor goes into the scale and the bias)
+    const float tau2 = -1.44269504089f * scale * (temp ? temp[h] : 1.0f), beta2 = bias ? -1.44269504089f * bias[h] : 0.0f;
     // this lane's operand of q: row r, values 32 st + 8 quad .. + 8
     sa_bf16x8 qreg[KS];
     const bf16* qrow = q + static_cast<size_t>(row0 + my_row) * ldq + static_cast<size_t>(h) * D;
@@ -216,7 +221,7 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_
             for (int i = 0; i < 4; ++i) {
                 const int key = kb + 16 * kt + 4 * quad + i;
                 const bool seen = key <= my_pos && (window <= 0 || key > my_pos - window);
-                w[kt][i] = static_cast<__bf16>(seen ? sa_sigmoid(sacc[kt][i] * tau + beta) : 0.0f);
+                w[kt][i] = static_cast<__bf16>(seen ? sa_sigmoid2(fmaf(sacc[kt][i], tau2, beta2)) : 0.0f);
             }
         // output, transposed: tile dt holds values 16 dt + 4 quad + i of row r
 #pragma unroll
@@ -296,7 +301,8 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_rows_
     const int my_pos = seq_start[s] + safe_row;
     const int wave_pos0 = seq_start[s] + first_row, wave_last = wave_pos0 + rows_here - 1;
     const int* pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
-    const float tau = scale * (temp ? temp[h] : 1.0f), beta = bias ? bias[h] : 0.0f;
+    // (sigmoid(x) = 1 / (1 + 2^(-x log2 e)): the factor goes into the scale and the bias)
+    const float tau2 = -1.44269504089f * scale * (temp ? temp[h] : 1.0f), beta2 = bias ? -1.44269504089f * bias[h] : 0.0f;
     sa_bf16x8 qreg[KS];
     const bf16* qrow = q + static_cast<size_t>(row0 + safe_row) * ldq + static_cast<size_t>(h) * D;
 #pragma unroll
@@ -373,7 +379,7 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_rows_
             for (int i = 0; i < 4; ++i) {
                 const int key = kb + 16 * kt + 4 * quad + i;
                 const bool seen = key <= my_pos && (window <= 0 || key > my_pos - window);
-                w[kt][i] = static_cast<__bf16>(seen ? sa_sigmoid(sacc[kt][i] * tau + beta) : 0.0f);
+                w[kt][i] = static_cast<__bf16>(seen ? sa_sigmoid2(fmaf(sacc[kt][i], tau2, beta2)) : 0.0f);
             }
 #pragma unroll
         for (int pair = 0; pair < 2; ++pair) {
