@@ -73,6 +73,70 @@ __global__ __launch_bounds__(256) void norm_step_kernel(float* __restrict__ h, c
     }
 }
 
+// The same for rows of up to 256 * NV values, with the row in registers and everything a thread reads
+// (branch output, stream, both norms' weights and biases) asked for at once: three trips to memory
+// one after the other become one, which is what a step of few rows waits for.
+template <int NV>
+__device__ __forceinline__ void reg_stats(const float (&v)[NV], const bool (&in)[NV], int width, int mode, float eps, float* scratch,
+                                          float& shift, float& factor) {
+    shift = 0.f;
+    factor = 1.f;
+    if (mode == CELEG_NORM_LAYER) {
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) s += in[k] ? v[k] : 0.f;
+        shift = block_sum(s, scratch) / static_cast<float>(width);
+    }
+    if (mode == CELEG_NORM_LAYER || mode == CELEG_NORM_RMS) {
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const float d = in[k] ? v[k] - shift : 0.f;
+            s += d * d;
+        }
+        factor = 1.0f / sqrtf(block_sum(s, scratch) / static_cast<float>(width) + eps);
+    }
+}
+
+template <typename TY, typename TO, int NV>
+__global__ __launch_bounds__(256) void norm_step_reg_kernel(float* __restrict__ h, const TY* __restrict__ y, CelegNorm post,
+                                                            CelegNorm pre, TO* __restrict__ out, const int* __restrict__ rows,
+                                                            int width, int write_back) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = static_cast<size_t>(rows ? rows[r] : r) * width;
+    float yv[NV], hv[NV], pw[NV], pb[NV], nw[NV], nb[NV];
+    bool in[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int i = threadIdx.x + 256 * k;
+        in[k] = i < width;
+        const int ii = in[k] ? i : 0;
+        hv[k] = h[src + ii];
+        yv[k] = y ? to_float(y[src + ii]) : 0.f;
+        pw[k] = y && post.w ? post.w[ii] : 1.f;
+        pb[k] = y && post.b ? post.b[ii] : 0.f;
+        nw[k] = out && pre.w ? pre.w[ii] : 1.f;
+        nb[k] = out && pre.b ? pre.b[ii] : 0.f;
+    }
+    if (y) {
+        float shift, factor;
+        reg_stats<NV>(yv, in, width, post.mode, post.eps, scratch, shift, factor);
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            hv[k] = ((yv[k] - shift) * factor * pw[k] + pb[k]) + hv[k];
+            if (write_back && in[k]) h[src + threadIdx.x + 256 * k] = hv[k];
+        }
+    }
+    if (!out) return;
+    float shift, factor;
+    reg_stats<NV>(hv, in, width, pre.mode, pre.eps, scratch, shift, factor);
+    TO* dst = out + static_cast<size_t>(r) * width;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+        if (in[k]) dst[threadIdx.x + 256 * k] = from_float<TO>((hv[k] - shift) * factor * nw[k] + nb[k]);
+}
+
 template <typename TO>
 __global__ void concat_rows_kernel(const float* __restrict__ a, const float* __restrict__ b, TO* __restrict__ out, size_t rows,
                                    int width) {
@@ -91,13 +155,20 @@ extern "C" int celeg_norm_step(float* h, const void* y, int y_dtype, CelegNorm p
     const size_t lds = static_cast<size_t>(width) * sizeof(float);
     if (lds > 60 * 1024) return static_cast<int>(hipErrorInvalidValue);
     dim3 grid(n_rows), block(256);
-#define CELEG_NORM_STEP(TY, TO)                                                                                    \
-    hipLaunchKernelGGL((norm_step_kernel<TY, TO>), grid, block, lds, stream, h, static_cast<const TY*>(y), post, pre, \
-                       static_cast<TO*>(out), rows, width, write_back)
-    if (y_dtype == CELEG_F32 && out_dtype == CELEG_F32) CELEG_NORM_STEP(float, float);
-    else if (y_dtype == CELEG_F32) CELEG_NORM_STEP(float, bf16);
-    else if (out_dtype == CELEG_F32) CELEG_NORM_STEP(bf16, float);
-    else CELEG_NORM_STEP(bf16, bf16);
+#define CELEG_NORM_STEP(TY, TO)                                                                                            \
+    if (width <= 1024)                                                                                                     \
+        hipLaunchKernelGGL((norm_step_reg_kernel<TY, TO, 4>), grid, block, 0, stream, h, static_cast<const TY*>(y), post, pre, \
+                           static_cast<TO*>(out), rows, width, write_back);                                               \
+    else if (width <= 2048)                                                                                                \
+        hipLaunchKernelGGL((norm_step_reg_kernel<TY, TO, 8>), grid, block, 0, stream, h, static_cast<const TY*>(y), post, pre, \
+                           static_cast<TO*>(out), rows, width, write_back);                                               \
+    else                                                                                                                   \
+        hipLaunchKernelGGL((norm_step_kernel<TY, TO>), grid, block, lds, stream, h, static_cast<const TY*>(y), post, pre,     \
+                           static_cast<TO*>(out), rows, width, write_back)
+    if (y_dtype == CELEG_F32 && out_dtype == CELEG_F32) { CELEG_NORM_STEP(float, float); }
+    else if (y_dtype == CELEG_F32) { CELEG_NORM_STEP(float, bf16); }
+    else if (out_dtype == CELEG_F32) { CELEG_NORM_STEP(bf16, float); }
+    else { CELEG_NORM_STEP(bf16, bf16); }
 #undef CELEG_NORM_STEP
     return CELEG_LAUNCH_RESULT();
 }

@@ -431,12 +431,13 @@ def test_gated_delta_rule_alone(tmp_path, H, G, D, V, taps):
     assert_close_f32(got, Wd["x"] + plain.gated_delta_rule(Wd["x"], m, Wd, "", 1e-4), "gated delta rule alone")
 
 
-@pytest.mark.parametrize("post", ["layernorm", "rmsnorm"])
-def test_norms_before_and_after_alone(tmp_path, post):
+@pytest.mark.parametrize("post,W_", [("layernorm", 36), ("rmsnorm", 36), ("layernorm", 1500), ("rmsnorm", 2304)])
+def test_norms_before_and_after_alone(tmp_path, post, W_):
     """No mixer (its output is zero, whose layer norm is the norm's bias), a dense feed-forward
-    between a layer norm and a norm of its output (a layer norm, or an RMS norm without bias)."""
+    between a layer norm and a norm of its output (a layer norm, or an RMS norm without bias).
+    Rows of up to 1,024, up to 2,048 and of more values take three forms of the kernel."""
     torch.manual_seed(3)
-    T, W_, ff = 29, 36, 40
+    T, ff = 29, 40
     t = {"x": torch.randn(T, W_) * 3 + 1, "g": torch.randn(ff, W_) * 0.3, "u": torch.randn(ff, W_) * 0.3, "d": torch.randn(W_, ff) * 0.3}
     for n in ("n1", "n1b", "n2", "n2b"):
         t[n], t[n + ".b"] = 1 + 0.3 * torch.randn(W_), torch.randn(W_) * 0.5
