@@ -346,6 +346,32 @@ def test_greedy_generation_through_the_entry_point(folders, name):
     engine.close()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_program(folders, tmp_path, dtype):
+    """``bin/trace_run`` in a process of its own: four schedules one after the other, a pool sized for
+    the live requests only, logits read from the files it writes."""
+    from helpers import TraceClient
+    folder = folders("K1", dtype)
+    reqs = requests_of("K1")
+    ref = plain_logits(folder, ("K1", dtype), reqs)
+    all_steps = []
+    for tag, make in (("w", whole_schedule), ("t", tail_decode_schedule), ("p", portions_schedule), ("m", mixed_schedule)):
+        for s in make({f"{tag}{rid}": toks for rid, toks in reqs.items()}):
+            all_steps.append(dict(s, step=len(all_steps)))
+    client = TraceClient(folder, dtype, str(tmp_path), peak_tokens(all_steps))
+    got = {}
+    for s in all_steps:
+        logits = client.step(s["step"], s["entries"], s["end"])
+        row = 0
+        for e in s["entries"]:
+            for _ in e["want"]:
+                got.setdefault(e["id"], []).append(torch.as_tensor(logits[row]))
+                row += 1
+    assert client.close() == 0
+    for rid_tagged, rows in got.items():
+        assert_close(torch.stack(rows), ref[rid_tagged[1:]], dtype, f"trace/{dtype}/{rid_tagged}")
+
+
 # ------------------------------------------------------------------ each mechanism alone
 def alone_architecture():
     """"KifetarPartsAlone": one block put together from what the configuration spells out; the
