@@ -87,7 +87,8 @@ __global__ __launch_bounds__(CELEG_WAVE) void sigmoid_attention_kernel(
 }
 
 // ---------------------------------------------------------------- bfloat16 on the matrix cores
-// One workgroup of four wavefronts per (16 rows of one request's step, query head).  The keys
+// One workgroup of four wavefronts (eight for heads of up to 64 values, whose staging areas fit)
+// per (16 rows of one request's step, query head).  The keys
 // the rows can see, from the first key of the first row's window (rounded down to 8, which stays
 // inside that key's page) to the last row's position, are walked in blocks of 64, the wavefronts
 // taking the blocks in turn and adding their sums at the end (a single token with a window of a
@@ -108,8 +109,8 @@ typedef unsigned int sa_u32x2 __attribute__((ext_vector_type(2)));
 #define SA_WAVES 4
 #define SA_KEYS 64
 
-template <int D>
-__global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_kernel(
+template <int D, int WAVES>
+__global__ __launch_bounds__(WAVES * CELEG_WAVE) void sigmoid_attention_mfma_kernel(
     const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
     const int* __restrict__ table, int table_stride, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_start, int n_seqs, const float* __restrict__ temp, const float* __restrict__ bias,
@@ -185,7 +186,7 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_
     };
     const int kb0 = (key_first & ~7) + wave * SA_KEYS;
     if (kb0 <= pos_last) fetch(kb0);
-    for (int kb = kb0; kb <= pos_last; kb += SA_WAVES * SA_KEYS) {
+    for (int kb = kb0; kb <= pos_last; kb += WAVES * SA_KEYS) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        if (kb + SA_WAVES * SA_KEYS <= pos_last) fetch(kb + SA_WAVES * SA_KEYS);
+        if (kb + WAVES * SA_KEYS <= pos_last) fetch(kb + WAVES * SA_KEYS);
         // scores, transposed: tile kt holds keys kb + 16 kt + 4 quad + i of row r
         sa_f32x4 sacc[4];
 #pragma unroll
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_mfma_
     __syncthreads();
     if (wave > 0 || r >= rows_here) return;
 #pragma unroll
-    for (int w = 1; w < SA_WAVES; ++w)
+    for (int w = 1; w < WAVES; ++w)
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -443,10 +444,12 @@ extern "C" int celeg_sigmoid_attention_fast(int form, const void* q, int ldq, co
     if (max_tiles <= 0 || n_seqs <= 0) return 0;
     if (!celeg_sigmoid_attention_fast_ok(head_dim) || q_heads % kv_heads || page_tokens % 8 || ldq % 8 || ldo % 4)
         return static_cast<int>(hipErrorInvalidValue);
-    dim3 grid(max_tiles, q_heads), block(SA_WAVES * CELEG_WAVE);
-    const size_t lds = static_cast<size_t>(form == 1 ? 2 : SA_WAVES) * (SA_KEYS * (head_dim + 8) + head_dim * (SA_KEYS + 8)) * 2;
+    // (single tiles: eight wavefronts share out the key blocks where their staging areas fit LDS)
+    const int waves = form == 1 ? SA_WAVES : head_dim <= 64 ? 8 : SA_WAVES;
+    dim3 grid(max_tiles, q_heads), block(waves * CELEG_WAVE);
+    const size_t lds = static_cast<size_t>(form == 1 ? 2 : waves) * (SA_KEYS * (head_dim + 8) + head_dim * (SA_KEYS + 8)) * 2;
 #define CELEG_SA_FAST(D_)                                                                                                        \
-    hipLaunchKernelGGL(form == 1 ? sigmoid_attention_rows_kernel<D_> : sigmoid_attention_mfma_kernel<D_>, grid, block, lds, stream, static_cast<const bf16*>(q), ldq,               \
+    hipLaunchKernelGGL((form == 1 ? sigmoid_attention_rows_kernel<D_> : sigmoid_attention_mfma_kernel<D_, (D_ <= 64 ? 8 : SA_WAVES)>), grid, block, lds, stream, static_cast<const bf16*>(q), ldq,               \
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table, table_stride, cu_seqlens, seq_slot, \
                        seq_start, n_seqs, temp, bias, static_cast<const bf16*>(gate), ldg, static_cast<bf16*>(out), ldo, q_heads,    \
                        kv_heads, page_tokens, n_layers, layer, scale, window)
