@@ -346,6 +346,26 @@ def test_greedy_generation_through_the_entry_point(folders, name):
     engine.close()
 
 
+def test_command_line(folders, tmp_path):
+    """``bin/celeg-run`` on a model folder of the design: greedy tokens and the prompt's last logits."""
+    import subprocess
+    import sys
+    import numpy as np
+    folder = folders("K2", "float32")
+    cfg, W = plain.load_model_folder(folder)
+    prompt = random_tokens(cfg["vocab"], 19, seed=5)
+    dump = str(tmp_path / "logits.f32")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "celeg-run"), "--model", folder, "--dtype", "float32", "--prompt",
+                           ",".join(map(str, prompt)), "--max-new-tokens", "8", "--repetition-penalty", "1.0", "--context", "128",
+                           "--runtime-tokens", "--dump-logits", dump], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr
+    line = [l for l in proc.stdout.splitlines() if l.startswith("CELEG_GENERATED_TOKEN_IDS=")][0]
+    assert json.loads(line.split("=", 1)[1]) == plain.greedy(cfg, W, prompt, 8)
+    logits = np.fromfile(dump, dtype="<f4")
+    assert_close_f32(torch.from_numpy(logits.copy()), plain.forward(cfg, W, prompt)[-1], "command line")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_replay_program(folders, tmp_path, dtype):
     """``bin/trace_run`` in a process of its own: four schedules one after the other, a pool sized for
