@@ -291,20 +291,39 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
         // them (one pass over S), u1 = b1 (v1 - a1 p1), u2 = b2 (v2 - a2 (a1 p2 + u1 k1.k2)),
         // o1 = a1 r1 + u1 k1.q1, o2 = a2 (a1 r2 + u1 k1.q2) + u2 k2.q2, and the state after them is
         // a2 a1 S + a2 u1 k1 + u2 k2 (a second pass): half as many passes that wait for one another.
-        auto two_tokens = [&](int tt, float v1, float v2) __attribute__((always_inline)) {
+        struct PairOperands {
+            f4 q1[NC], k1[NC], q2[NC], k2[NC];
+            float b1, a1, b2, a2, k1k2, k1q1, k1q2, k2q2;
+        };
+        // (a pair's operands are read from LDS while the pair before is computed)
+        auto read_pair = [&](int tt) __attribute__((always_inline)) {
+            PairOperands p;
             const float* row1 = qk_s + tt * ROW + sub * DPL;
             const float* row2 = row1 + ROW;
-            f4 q1[NC], k1[NC], q2[NC], k2[NC];
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                q1[c] = *reinterpret_cast<const f4*>(row1 + 4 * c);
-                k1[c] = *reinterpret_cast<const f4*>(row1 + D + 4 * c);
-                q2[c] = *reinterpret_cast<const f4*>(row2 + 4 * c);
-                k2[c] = *reinterpret_cast<const f4*>(row2 + D + 4 * c);
+                p.q1[c] = *reinterpret_cast<const f4*>(row1 + 4 * c);
+                p.k1[c] = *reinterpret_cast<const f4*>(row1 + D + 4 * c);
+                p.q2[c] = *reinterpret_cast<const f4*>(row2 + 4 * c);
+                p.k2[c] = *reinterpret_cast<const f4*>(row2 + D + 4 * c);
             }
-            const float b1 = bd_s[2 * tt], a1 = bd_s[2 * tt + 1], b2 = bd_s[2 * tt + 2], a2 = bd_s[2 * tt + 3];
+            p.b1 = bd_s[2 * tt];
+            p.a1 = bd_s[2 * tt + 1];
+            p.b2 = bd_s[2 * tt + 2];
+            p.a2 = bd_s[2 * tt + 3];
             const float* ps = pair_s + 2 * tt;
-            const float k1k2 = ps[0], k1q1 = ps[1], k1q2 = ps[2], k2q2 = ps[3];
+            p.k1k2 = ps[0];
+            p.k1q1 = ps[1];
+            p.k1q2 = ps[2];
+            p.k2q2 = ps[3];
+            return p;
+        };
+        auto two_tokens = [&](int tt, const PairOperands& p, float v1, float v2) __attribute__((always_inline)) {
+            const f4 (&q1)[NC] = p.q1;
+            const f4 (&k1)[NC] = p.k1;
+            const f4 (&q2)[NC] = p.q2;
+            const f4 (&k2)[NC] = p.k2;
+            const float b1 = p.b1, a1 = p.a1, b2 = p.b2, a2 = p.a2, k1k2 = p.k1k2, k1q1 = p.k1q1, k1q2 = p.k1q2, k2q2 = p.k2q2;
             float p1[2] = {0.f, 0.f}, p2[2] = {0.f, 0.f}, r1[2] = {0.f, 0.f}, r2[2] = {0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < NC; ++c)
@@ -336,8 +355,14 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
         if (count == TB && pairs) {
             // a whole block: one run of instructions, so that the next tokens' operands are read while
             // these are computed
+            PairOperands now = read_pair(0);
 #pragma unroll
-            for (int tt = 0; tt < TB; tt += 2) two_tokens(tt, vals[tt], vals[tt + 1]);
+            for (int tt = 0; tt < TB; tt += 2) {
+                PairOperands next = now;
+                if (tt + 2 < TB) next = read_pair(tt + 2);
+                two_tokens(tt, now, vals[tt], vals[tt + 1]);
+                now = next;
+            }
         } else if (count == TB) {
 #pragma unroll
             for (int tt = 0; tt < TB; ++tt) token(tt, vals[tt]);

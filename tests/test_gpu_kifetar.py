@@ -178,7 +178,7 @@ def test_batches_of_unequal_requests_equal_each_alone(folders):
 
 
 # ------------------------------------------------------------------ weights made so that a fault shows
-WINDOWS = (1, 2, 16, 17, 31)
+WINDOWS = (1, 2, 16, 17, 31, None)      # (None: every earlier key, however far)
 
 
 def windows_model(windows=WINDOWS):
@@ -212,8 +212,8 @@ def test_a_window_one_key_off_shows():
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_window_edges_in_prompts_and_decoding(tmp_path, dtype):
-    """Windows of 1, 2, 16 (a page), 17 and 31 keys with sharp weights, in whole prompts, in portions
-    of every size and in tokens decoded one by one past every window's length."""
+    """Windows of 1, 2, 16 (a page), 17 and 31 keys and no window at all, with sharp weights, in whole
+    prompts, in portions of every size and in tokens decoded one by one past every window's length."""
     cfg = windows_model()
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = write_model(tmp_path / "win", cfg, 5, storage, std=0.1, change=sharp(cfg, 6.0 if dtype == "float32" else 2.0))
