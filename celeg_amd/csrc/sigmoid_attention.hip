@@ -151,6 +151,8 @@ __global__ __launch_bounds__(WAVES * CELEG_WAVE) void sigmoid_attention_mfma_ker
     for (int dt = 0; dt < DT; ++dt) oacc[dt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
     const int key_first = window > 0 ? max(0, pos0 - window + 1) : 0;
     const size_t head_stride = static_cast<size_t>(page_tokens) * D;
+    // (pages hold a power of two of tokens here: a key's page and place by a shift and a mask, not a division)
+    const int page_shift = 31 - __builtin_clz(page_tokens), page_mask = page_tokens - 1;
     constexpr int KCH = SA_KEYS * (D / 8) / CELEG_WAVE, VCH = D * (SA_KEYS / 8) / CELEG_WAVE;   // 16-byte pieces a lane
     sa_u32x4 kpre[KCH], vpre[VCH];
     // a block's pieces from memory into registers: keys kb .. kb + 63 (those past pos_last: the last
@@ -160,8 +162,8 @@ __global__ __launch_bounds__(WAVES * CELEG_WAVE) void sigmoid_attention_mfma_ker
         for (int i = 0; i < KCH; ++i) {
             const int c = lane + CELEG_WAVE * i, key_in = c / (D / 8), part = c % (D / 8);
             const int key = min(kb + key_in, pos_last);
-            const bf16* src = k_pool + ((static_cast<size_t>(pages[key / page_tokens]) * n_layers + layer) * kv_heads + kvh) * head_stride +
-                              static_cast<size_t>(key % page_tokens) * D + 8 * part;
+            const bf16* src = k_pool + ((static_cast<size_t>(pages[key >> page_shift]) * n_layers + layer) * kv_heads + kvh) * head_stride +
+                              static_cast<size_t>((key & page_mask)) * D + 8 * part;
             kpre[i] = *reinterpret_cast<const sa_u32x4*>(src);
         }
 #pragma unroll
@@ -170,8 +172,8 @@ __global__ __launch_bounds__(WAVES * CELEG_WAVE) void sigmoid_attention_mfma_ker
             const int key = kb + 8 * part;         // eight keys that lie side by side in one page
             sa_u32x4 val = {0u, 0u, 0u, 0u};
             if (key <= pos_last) {
-                const bf16* src = v_pool + ((static_cast<size_t>(pages[key / page_tokens]) * n_layers + layer) * kv_heads + kvh) * head_stride +
-                                  static_cast<size_t>(d) * page_tokens + key % page_tokens;
+                const bf16* src = v_pool + ((static_cast<size_t>(pages[key >> page_shift]) * n_layers + layer) * kv_heads + kvh) * head_stride +
+                                  static_cast<size_t>(d) * page_tokens + (key & page_mask);
                 val = *reinterpret_cast<const sa_u32x4*>(src);
                 const int live = pos_last - key + 1;       // keys of this piece that exist
                 if (live < 8) {
@@ -313,14 +315,16 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_rows_
     for (int dt = 0; dt < DT; ++dt) oacc[dt] = sa_f32x4{0.f, 0.f, 0.f, 0.f};
     const int key_first = window > 0 ? max(0, tile_pos0 - window + 1) : 0;
     const size_t head_stride = static_cast<size_t>(page_tokens) * D;
+    // (pages hold a power of two of tokens here: a key's page and place by a shift and a mask, not a division)
+    const int page_shift = 31 - __builtin_clz(page_tokens), page_mask = page_tokens - 1;
     sa_u32x4 kpre[KCH], vpre[VCH];
     auto fetch = [&](int kb) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < KCH; ++i) {
             const int c = tid + THREADS * i, key_in = c / (D / 8), part = c % (D / 8);
             const int key = min(kb + key_in, pos_last);
-            const bf16* src = k_pool + ((static_cast<size_t>(pages[key / page_tokens]) * n_layers + layer) * kv_heads + kvh) * head_stride +
-                              static_cast<size_t>(key % page_tokens) * D + 8 * part;
+            const bf16* src = k_pool + ((static_cast<size_t>(pages[key >> page_shift]) * n_layers + layer) * kv_heads + kvh) * head_stride +
+                              static_cast<size_t>((key & page_mask)) * D + 8 * part;
             kpre[i] = *reinterpret_cast<const sa_u32x4*>(src);
         }
 #pragma unroll
@@ -329,8 +333,8 @@ __global__ __launch_bounds__(SA_WAVES * CELEG_WAVE) void sigmoid_attention_rows_
             const int key = kb + 8 * part;
             sa_u32x4 val = {0u, 0u, 0u, 0u};
             if (key <= pos_last) {
-                const bf16* src = v_pool + ((static_cast<size_t>(pages[key / page_tokens]) * n_layers + layer) * kv_heads + kvh) * head_stride +
-                                  static_cast<size_t>(d) * page_tokens + key % page_tokens;
+                const bf16* src = v_pool + ((static_cast<size_t>(pages[key >> page_shift]) * n_layers + layer) * kv_heads + kvh) * head_stride +
+                                  static_cast<size_t>(d) * page_tokens + (key & page_mask);
                 val = *reinterpret_cast<const sa_u32x4*>(src);
                 const int live = pos_last - key + 1;
                 if (live < 8) {
@@ -442,7 +446,8 @@ extern "C" int celeg_sigmoid_attention_fast(int form, const void* q, int ldq, co
                                             int ldg, void* out, int ldo, int q_heads, int kv_heads, int head_dim, int page_tokens,
                                             int n_layers, int layer, float scale, int window, hipStream_t stream) {
     if (max_tiles <= 0 || n_seqs <= 0) return 0;
-    if (!celeg_sigmoid_attention_fast_ok(head_dim) || q_heads % kv_heads || page_tokens % 8 || ldq % 8 || ldo % 4)
+    if (!celeg_sigmoid_attention_fast_ok(head_dim) || q_heads % kv_heads || page_tokens % 8 || (page_tokens & (page_tokens - 1)) ||
+        ldq % 8 || ldo % 4)
         return static_cast<int>(hipErrorInvalidValue);
     // (single tiles: eight wavefronts share out the key blocks where their staging areas fit LDS)
     const int waves = form == 1 ? SA_WAVES : head_dim <= 64 ? 8 : SA_WAVES;
